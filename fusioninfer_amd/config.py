@@ -42,6 +42,11 @@ class ModelConfig:
     num_experts_per_tok: int = 8
     moe_intermediate_size: int = 0
     norm_topk_prob: bool = True
+    # model family: "transformer" is the Llama/Qwen decoder (CausalLM);
+    # other families are registered in models/registry.py and carry their
+    # own parsed description in `arch` (layer list, mixer constants)
+    architecture: str = "transformer"
+    arch: Optional[object] = None
 
     @property
     def is_moe(self) -> bool:
@@ -142,3 +147,6 @@ class EngineConfig:
     max_cpu_loras: int = 16
     seed: int = 0
     enforce_eager: bool = False            # True disables hipGraph decode capture
+    # state slots for models with per-sequence recurrent state (one slot
+    # per live sequence); None = scheduler.max_num_seqs
+    num_state_slots: Optional[int] = None

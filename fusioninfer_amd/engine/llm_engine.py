@@ -71,12 +71,32 @@ class LLMEngine:
         self.device = device
         self.runner = ModelRunner(cfg, device)
         self.runner.allocate_kv_caches()
+        self.state_manager = None
+        if self.runner.uses_state_slots:
+            # recurrent per-sequence state: one slot per live sequence.
+            # Features that move or share cache blocks without the state
+            # (prefix reuse, host swap, KV export, draft verification
+            # that would have to roll the state back) are off.
+            from fusioninfer_amd.engine.state_manager import StateSlotManager
+
+            self.state_manager = StateSlotManager(self.runner.num_state_slots)
+            cfg.cache.enable_prefix_caching = False
+            if cfg.cache.swap_space_gb > 0:
+                raise ValueError("--swap-space is not supported for models "
+                                 "with recurrent state")
+            if cfg.speculative is not None:
+                raise ValueError("speculative decoding is not supported for "
+                                 "models with recurrent state")
+            if cfg.kv_transfer.kv_connector:
+                raise ValueError("PD disaggregation is not supported for "
+                                 "models with recurrent state")
         self.block_manager = BlockManager(
             self.runner.num_gpu_blocks,
             cfg.cache.block_size,
             enable_prefix_caching=cfg.cache.enable_prefix_caching,
         )
-        self.scheduler = Scheduler(cfg.scheduler, self.block_manager)
+        self.scheduler = Scheduler(cfg.scheduler, self.block_manager,
+                                   self.state_manager)
         self._swapped: Dict[str, "torch.Tensor"] = {}
         self._swap_bytes = 0
         self.num_swap_outs = 0
@@ -101,6 +121,8 @@ class LLMEngine:
         self.runner.capture_decode_graphs()
         self._req_counter = itertools.count()
         self.seqs: Dict[str, Sequence] = {}
+        # requests driven through forced_step (not owned by the scheduler)
+        self._forced: Dict[str, Sequence] = {}
         self._held: Dict[str, Sequence] = {}
         # PD: the KV connector (set by the server/pd wiring on every TP
         # rank; worker ranks use it for pd_send / pd_recv commands)
@@ -292,6 +314,8 @@ class LLMEngine:
             self.block_manager.free(seq)
         elif seq.block_ids:
             self.block_manager.free(seq)
+        if self.state_manager is not None:
+            self.state_manager.free(seq)
         seq.status = SeqStatus.FINISHED
         return True
 
@@ -761,6 +785,7 @@ class LLMEngine:
             "lens": [s.num_tokens + 1 for s in keep],
             "bt": [list(s.block_ids) for s in keep],
             "lora_names": [None] * len(keep),
+            "state_slots": [s.state_slot for s in keep],
         }
         sampled = p["sampled"]
         if len(keep) != len(p["seqs"]):
@@ -955,6 +980,106 @@ class LLMEngine:
                     # accepted prefix (no-op for ngram)
                     self.proposer.commit(s, m)
         return outputs
+
+    # ------------------------------------------------------- forced steps
+    def forced_step(self, entries, end=()):
+        """Teacher-forced step: run GIVEN next tokens of several requests
+        as one batch and return logits at chosen places. Nothing is
+        sampled; the caller decides what each request sees next.
+
+        entries: [(request_id, tokens, want)] - `tokens` continue the
+        request (it is admitted at its first entry), `want` lists indices
+        into `tokens` whose logits are returned. `end`: requests to
+        release after the step. Returns fp32 logits [sum(len(want)), V] in
+        the order of entries and want.
+
+        This is the engine's own step underneath: blocks and state slots
+        come from the block/state managers, a continuation of exactly one
+        token rides the decode segment (hipGraph replay when the whole
+        step is decode), longer portions the chunked-prefill segment, and
+        the model runner executes them as one mixed batch. Used for
+        scoring and for replaying recorded schedules."""
+        assert self.is_driver and self.exec_world_size() == 1
+        if self._pending is not None:
+            self._drained_backlog.extend(self._drain_pending())
+        bm = self.block_manager
+        held = self._forced
+        if not entries:
+            for rid in end:
+                seq = held.pop(rid, None)
+                if seq is not None:
+                    bm.free(seq)
+                    if self.state_manager is not None:
+                        self.state_manager.free(seq)
+                    seq.status = SeqStatus.FINISHED
+            return torch.empty((0, self.cfg.model.vocab_size))
+        prefill, chunks, decode = [], [], []
+        need = 0
+        for rid, tokens, _ in entries:
+            seq = held.get(rid)
+            n_old = seq.num_prompt_tokens if seq is not None else 0
+            have = len(seq.block_ids) if seq is not None else 0
+            need += max(bm.blocks_needed(n_old + len(tokens)) - have, 0)
+        if need > bm.num_free():
+            raise InsufficientBlocksError(
+                f"forced step needs {need} cache blocks, "
+                f"{bm.num_free()} free")
+        for rid, tokens, _ in entries:
+            if not tokens:
+                raise ValueError(f"request {rid!r}: empty continuation")
+            seq = held.get(rid)
+            if seq is None:
+                seq = Sequence(rid, [], SamplingParams())
+                if self.state_manager is not None:
+                    self.state_manager.allocate(seq)
+                seq.status = SeqStatus.RUNNING
+                held[rid] = seq
+            done = seq.num_prompt_tokens
+            seq.prompt_token_ids.extend(int(t) for t in tokens)
+            if seq.num_prompt_tokens > self.cfg.scheduler.max_model_len:
+                raise ValueError(f"request {rid!r} exceeds max_model_len")
+            bm.append_slots_upto(seq, seq.num_prompt_tokens - 1)
+            seq.num_computed_tokens = done
+            if len(tokens) == 1 and done > 0:
+                decode.append(seq)
+            else:
+                prefill.append(seq)
+                chunks.append(len(tokens))
+        payload = self.runner.build_batch_payload(prefill, chunks, decode, bm)
+        # payload rows: prefill chunks in order, then the decode rows
+        row0 = {}
+        for seq, c0 in zip(prefill, payload["cu"]):
+            row0[seq.seq_id] = c0
+        for i, seq in enumerate(decode):
+            row0[seq.seq_id] = payload["cu"][-1] + i
+        asked = [row0[rid] + int(w) for rid, tokens, want in entries
+                 for w in want]
+        for rid, tokens, want in entries:
+            if any(not 0 <= int(w) < len(tokens) for w in want):
+                raise ValueError(f"request {rid!r}: want outside its tokens")
+        rows = sorted(set(asked))
+        pure_decode = not prefill
+        if not pure_decode:
+            payload["logits_rows"] = rows
+        logits = self.runner.run_batch(payload)
+        if pure_decode:
+            at = {r: r for r in range(len(decode))}
+        else:
+            at = {r: i for i, r in enumerate(rows)}
+        out = logits.float()[[at[r] for r in asked]] if asked else \
+            logits.float()[:0]
+        for seq in prefill + decode:
+            seq.num_computed_tokens = seq.num_prompt_tokens
+        self.num_prefilled_tokens += sum(chunks) + len(decode)
+        for rid in end:
+            seq = held.pop(rid, None)
+            if seq is None:
+                continue
+            bm.free(seq)
+            if self.state_manager is not None:
+                self.state_manager.free(seq)
+            seq.status = SeqStatus.FINISHED
+        return out
 
     # --------------------------------------------------------- TP workers
     def worker_loop(self) -> None:

@@ -28,6 +28,13 @@ class AttnMetadata:
     # decode segment
     block_tables: Optional[torch.Tensor] = None  # [Dq, max_blocks] int32
     seq_lens: Optional[torch.Tensor] = None      # [Dq] int32 (ctx incl. current)
+    # sequence-grouped view of ALL rows (models with per-sequence state or
+    # per-row key ranges): prefill groups first, then one-row decode groups
+    seq_cu: Optional[torch.Tensor] = None        # [S+1] int32 row offsets
+    row_seq: Optional[torch.Tensor] = None       # [T] int32 group of a row
+    seq_bt: Optional[torch.Tensor] = None        # [S, max_blocks] int32
+    seq_slots: Optional[torch.Tensor] = None     # [S] int32 state slot (-1 none)
+    max_seq_rows: int = 0                        # longest group (host int)
     # LoRA groups for this step (fusioninfer_amd.lora.LoRABatch) or None
     lora: object = None
 

@@ -25,7 +25,7 @@ from fusioninfer_amd.config import EngineConfig
 from fusioninfer_amd.engine.block_manager import BlockManager
 from fusioninfer_amd.engine.metadata import AttnMetadata
 from fusioninfer_amd.engine.sequence import Sequence
-from fusioninfer_amd.models.model import CausalLM
+from fusioninfer_amd.models.registry import build_model
 import fusioninfer_amd.ops as ops_mod
 
 _DECODE_BUCKETS = [1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 160, 192, 224, 256, 320, 384, 448, 512]
@@ -48,7 +48,14 @@ class ModelRunner:
                 # auto-detects this from quantization_config too)
                 mc.quantization = "fp8"
         with torch.device(self.device):
-            self.model = CausalLM(mc).eval()
+            self.model = build_model(mc).eval()
+        # models with per-sequence recurrent state (state slots) and
+        # per-row key ranges read a sequence-grouped view of the batch
+        self.uses_state_slots = bool(
+            getattr(self.model, "uses_state_slots", False))
+        self.num_state_slots = (
+            (cfg.num_state_slots or cfg.scheduler.max_num_seqs)
+            if self.uses_state_slots else 0)
         if mc.quantization == "fp8" and fp8_ckpt:
             # fp8-native checkpoint: convert modules FIRST (fp8 storage +
             # scale buffers exist), then load e4m3 weights + weight_scale
@@ -98,6 +105,9 @@ class ModelRunner:
         mc = self.cfg.model
         import fusioninfer_amd.distributed.parallel_state as ps
 
+        if hasattr(self.model, "kv_block_bytes"):
+            # the family declares its own per-run cache shapes
+            return self.model.kv_block_bytes(self.block_size)
         kv_heads = mc.num_kv_heads // ps.tp_world_size()
         esize = 1 if self.cfg.cache.kv_cache_dtype == "fp8" else 2
         layers = self.model.num_local_layers  # PP stages hold a layer slice
@@ -126,6 +136,12 @@ class ModelRunner:
 
         mc = self.cfg.model
         self.num_gpu_blocks = self.profile_num_blocks()
+        if hasattr(self.model, "allocate_caches"):
+            # per layer RUN: paged tensors plus slot-indexed state tensors
+            self.kv_caches = self.model.allocate_caches(
+                self.num_gpu_blocks, self.block_size, self.num_state_slots,
+                self.device)
+            return
         kv_heads = mc.num_kv_heads // ps.tp_world_size()
         shape = (self.num_gpu_blocks, kv_heads, self.block_size, mc.head_dim)
         kv_dtype = (
@@ -196,7 +212,39 @@ class ModelRunner:
             "bt": bt,
             "sample": sample,
             "lora_names": [s.lora_name for s in seqs],
+            "state_slots": [s.state_slot for s in seqs],
         }
+
+    def _seq_meta(self, meta: AttnMetadata, prefill_payload, decode_payload):
+        """Sequence-grouped view of the step for models with state slots:
+        prefill chunks as multi-row groups, then one-row decode groups."""
+        if not self.uses_state_slots:
+            return meta
+        dev = self.device
+        lens, slots, bts = [], [], []
+        if prefill_payload is not None and prefill_payload["new_lens"]:
+            lens += list(prefill_payload["new_lens"])
+            slots += list(prefill_payload["state_slots"])
+            bts += [list(b) for b in prefill_payload["bt"]]
+        if decode_payload is not None and decode_payload["lens"]:
+            n = len(decode_payload["lens"])
+            lens += [1] * n
+            slots += list(decode_payload["state_slots"])
+            bts += [list(b) for b in decode_payload["bt"]]
+        S = len(lens)
+        cu = np.zeros(S + 1, dtype=np.int32)
+        np.cumsum(np.asarray(lens, dtype=np.int32), out=cu[1:])
+        width = max(max((len(b) for b in bts), default=1), 1)
+        bt_np = np.zeros((S, width), dtype=np.int32)
+        for i, b in enumerate(bts):
+            bt_np[i, : len(b)] = b
+        meta.seq_cu = torch.from_numpy(cu).to(dev)
+        meta.row_seq = torch.from_numpy(
+            np.repeat(np.arange(S, dtype=np.int32), lens)).to(dev)
+        meta.seq_bt = torch.from_numpy(bt_np).to(dev)
+        meta.seq_slots = torch.tensor(slots, dtype=torch.int32, device=dev)
+        meta.max_seq_rows = max(lens, default=0)
+        return meta
 
     def _lora_batch(self, prefill_payload, decode_payload, np_=0):
         """Group this step's token rows by adapter -> LoRABatch or None."""
@@ -267,6 +315,7 @@ class ModelRunner:
             ),
         )
         meta.lora = self._lora_batch(payload, None)
+        self._seq_meta(meta, payload, None)
         ids = torch.tensor(payload["ids"], dtype=torch.long, device=dev)
         if payload.get("logits_rows") is not None:
             # spec-decode verification asks for explicit rows (every draft
@@ -464,13 +513,14 @@ class ModelRunner:
             if prefill_seqs
             else {"kind": "prefill", "ids": [], "positions": [], "slots": [],
                   "cu": [0], "new_lens": [], "total_lens": [], "bt": [],
-                  "sample": []}
+                  "sample": [], "state_slots": []}
         )
         payload["kind"] = "mixed"
         d = (
             self.build_decode_payload(decode_seqs, bm)
             if decode_seqs
-            else {"ids": [], "positions": [], "slots": [], "lens": [], "bt": []}
+            else {"ids": [], "positions": [], "slots": [], "lens": [], "bt": [],
+                  "state_slots": []}
         )
         payload["decode"] = d
         return payload
@@ -544,6 +594,7 @@ class ModelRunner:
             "sample": sample,
             "logits_rows": logits_rows,
             "lora_names": [s.lora_name for s in all_seqs],
+            "state_slots": [s.state_slot for s in all_seqs],
         }
 
     def run_batch(self, payload) -> torch.Tensor:
@@ -590,6 +641,7 @@ class ModelRunner:
             seq_lens=torch.tensor(d["lens"], dtype=torch.int32, device=dev),
         )
         meta.lora = self._lora_batch(payload, d, np_=np_)
+        self._seq_meta(meta, payload, d)
         ids = torch.tensor(
             payload["ids"] + d["ids"], dtype=torch.long, device=dev
         )
@@ -624,6 +676,14 @@ class ModelRunner:
             ),
             "seq_lens": torch.ones(max_bs, dtype=torch.int32, device=dev),
         }
+        if self.uses_state_slots:
+            # every decode row is its own one-row group
+            self._static["state_slots"] = torch.full(
+                (max_bs,), -1, dtype=torch.int32, device=dev)
+            self._static["seq_cu"] = torch.arange(
+                max_bs + 1, dtype=torch.int32, device=dev)
+            self._static["row_seq"] = torch.arange(
+                max_bs, dtype=torch.int32, device=dev)
 
     def _decode_forward(self, bs: int, lora=None) -> torch.Tensor:
         s = self._static
@@ -636,6 +696,12 @@ class ModelRunner:
             block_tables=s["block_tables"][:bs],
             seq_lens=s["seq_lens"][:bs],
         )
+        if self.uses_state_slots:
+            meta.seq_cu = s["seq_cu"][: bs + 1]
+            meta.row_seq = s["row_seq"][:bs]
+            meta.seq_bt = s["block_tables"][:bs]
+            meta.seq_slots = s["state_slots"][:bs]
+            meta.max_seq_rows = 1
         return self._forward_and_logits(
             s["ids"][:bs], meta,
             torch.arange(bs, dtype=torch.long, device=self.device),
@@ -680,6 +746,7 @@ class ModelRunner:
             "lens": [s.num_tokens for s in seqs],
             "bt": [list(s.block_ids) for s in seqs],
             "lora_names": [s.lora_name for s in seqs],
+            "state_slots": [s.state_slot for s in seqs],
         }
 
     def _fill_decode_inputs(self, payload, bs: int) -> None:
@@ -709,6 +776,13 @@ class ModelRunner:
         st["block_tables"][:n].copy_(
             torch.from_numpy(bt_np), non_blocking=True
         )
+        if self.uses_state_slots:
+            st["state_slots"][:n].copy_(
+                torch.tensor(payload["state_slots"], dtype=torch.int32),
+                non_blocking=True,
+            )
+            if bs > n:
+                st["state_slots"][n:bs].fill_(-1)
         if bs > n:  # padding rows: decode block 0, pos 0, len 1, slot -1
             st["ids"][n:bs].zero_()
             st["positions"][n:bs].zero_()

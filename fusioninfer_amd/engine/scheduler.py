@@ -51,9 +51,14 @@ class Scheduler:
     #: adaptive admission window = this many steps of EMA step time
     ADMISSION_STEPS = 4.0
 
-    def __init__(self, cfg: SchedulerConfig, block_manager: BlockManager):
+    def __init__(self, cfg: SchedulerConfig, block_manager: BlockManager,
+                 state_manager=None):
         self.cfg = cfg
         self.bm = block_manager
+        # engine/state_manager.StateSlotManager for models with recurrent
+        # per-sequence state: a sequence holds one slot from admission to
+        # finish/preemption (re-prefill rebuilds the state from position 0)
+        self.sm = state_manager
         self._step_ema_s = 0.05  # updated by the engine after each step
         self.waiting: Deque[Sequence] = deque()
         self.running: List[Sequence] = []
@@ -209,6 +214,10 @@ class Scheduler:
                 break
             if not self.bm.can_allocate(seq.num_prompt_tokens):
                 break
+            if self.sm is not None:
+                if not self.sm.can_allocate():
+                    break
+                self.sm.allocate(seq)
             self.waiting.popleft()
             self.bm.allocate(seq)
             seq.status = SeqStatus.RUNNING
@@ -237,6 +246,8 @@ class Scheduler:
             self.waiting.appendleft(victim)
             return victim
         self.bm.free(victim)
+        if self.sm is not None:
+            self.sm.free(victim)
         victim.status = SeqStatus.PREEMPTED
         # recompute: generated tokens become part of the prompt
         victim.prompt_token_ids.extend(victim.output_token_ids)
@@ -251,4 +262,6 @@ class Scheduler:
         seq.status = SeqStatus.FINISHED
         if not seq.hold_blocks:
             self.bm.free(seq)
+        if self.sm is not None:
+            self.sm.free(seq)
         self.running.remove(seq)

@@ -85,6 +85,9 @@ class Sequence:
         # stop token / grammar terminal); None while running
         self.finish_reason = None
         self.swap_num_blocks = 0
+        # slot in the runner's per-sequence state tensors (models with
+        # recurrent mixers); -1 = none held
+        self.state_slot = -1
         # LoRA adapter name (None = base model)
         self.lora_name = None
         # scheduling priority (lower = more urgent; "priority" policy)

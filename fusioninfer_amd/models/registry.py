@@ -201,7 +201,83 @@ register(
 )
 
 
+# ------------------------------------------------------- architectures
+#
+# A model FAMILY beyond the built-in transformer registers (a) how its
+# config.json becomes a ModelConfig and (b) which module class the model
+# runner instantiates. Checkpoint directories select the family by the
+# "architecture" key of their config.json.
+
+_ARCHITECTURES = {}
+
+
+def register_architecture(name: str, config_from_dict, model_factory) -> None:
+    """config_from_dict(raw: dict, model_path) -> ModelConfig;
+    model_factory(cfg: ModelConfig) -> nn.Module."""
+    _ARCHITECTURES[name.lower()] = (config_from_dict, model_factory)
+
+
+def _register_builtin_architectures() -> None:
+    def pinuvik_config(raw, model_path):
+        from fusioninfer_amd.models import pinuvik
+
+        return pinuvik.model_config_from_dict(raw, model_path)
+
+    def pinuvik_model(cfg):
+        from fusioninfer_amd.models.pinuvik import PinuvikLM
+
+        return PinuvikLM(cfg)
+
+    register_architecture("Pinuvik", pinuvik_config, pinuvik_model)
+
+
+_register_builtin_architectures()
+
+
+def model_config_from_dir(path: str) -> ModelConfig:
+    """ModelConfig for a checkpoint directory whose config.json names a
+    registered architecture."""
+    import json
+    import os
+
+    with open(os.path.join(path, "config.json")) as f:
+        raw = json.load(f)
+    arch = str(raw.get("architecture", "")).lower()
+    if arch not in _ARCHITECTURES:
+        raise KeyError(
+            f"config.json architecture {raw.get('architecture')!r} is not "
+            f"registered; known: {sorted(_ARCHITECTURES)}")
+    has_weights = any(f.endswith(".safetensors") for f in os.listdir(path))
+    return _ARCHITECTURES[arch][0](raw, path if has_weights else None)
+
+
+def model_config_from_dict(raw: dict) -> ModelConfig:
+    """Random-init ModelConfig from an in-memory config dict."""
+    arch = str(raw.get("architecture", "")).lower()
+    if arch not in _ARCHITECTURES:
+        raise KeyError(f"architecture {raw.get('architecture')!r} is not "
+                       f"registered; known: {sorted(_ARCHITECTURES)}")
+    return _ARCHITECTURES[arch][0](raw, None)
+
+
+def build_model(cfg: ModelConfig):
+    """Instantiate the module class of cfg's family."""
+    if cfg.architecture == "transformer":
+        from fusioninfer_amd.models.model import CausalLM
+
+        return CausalLM(cfg)
+    key = cfg.architecture.lower()
+    if key not in _ARCHITECTURES:
+        raise KeyError(f"unknown architecture {cfg.architecture!r}")
+    return _ARCHITECTURES[key][1](cfg)
+
+
 def get_model_config(name: str) -> ModelConfig:
+    import os as _os
+
+    if _os.path.isdir(name) and _os.path.exists(
+            _os.path.join(name, "config.json")):
+        return model_config_from_dir(name)
     key = name.lower()
     if key not in _REGISTRY and "/" in key:
         # accept HF-style ids ("Qwen/Qwen3-8B" -> "Qwen3-8B")

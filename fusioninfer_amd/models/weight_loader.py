@@ -334,6 +334,9 @@ def load_safetensors_dir(model, path: str) -> int:
                 for name in sf.keys():
                     yield name, sf.get_tensor(name)
 
+    if hasattr(model, "load_weights"):
+        # families outside the HF transformer layout map their own names
+        return model.load_weights(tensor_iter())
     return load_hf_state_dict(model, tensor_iter())
 
 

@@ -3,7 +3,12 @@
 Drives hipcc directly — no CUDA compatibility layer, no JIT cache: the
 resulting ``_C.so`` lives next to this file so the gpurun snapshot carries it.
 
-Usage:  python -m fusioninfer_amd.ops.build
+Two extensions, so that a model family compiles only what it runs:
+
+  core    -> _C.so         transformer / MoE kernels
+  seqmix  -> _C_seqmix.so  sequence-mixer kernels (ops/seqmix.py)
+
+Usage:  python -m fusioninfer_amd.ops.build [core|seqmix|all] [--force]
 """
 
 from __future__ import annotations
@@ -30,16 +35,44 @@ SOURCES = [
 ]
 
 
+SEQMIX_SOURCES = [
+    "seqmix_bindings.hip",
+    "seqmix_norm.hip",
+    "seqmix_attention.hip",
+    "seqmix_delta.hip",
+]
+
+EXTENSIONS = {
+    "core": ("_C", SOURCES, ["common.h"]),
+    "seqmix": ("_C_seqmix", SEQMIX_SOURCES, ["common.h", "seqmix.h"]),
+}
+
+
+def extension_path(ext: str) -> str:
+    return os.path.join(OPS_DIR, EXTENSIONS[ext][0] + ".so")
+
+
 def build(verbose: bool = True, force: bool = False) -> str:
+    """The core extension (kept as the historical entry point)."""
+    return build_extension("core", verbose=verbose, force=force)
+
+
+def build_extension(ext: str, verbose: bool = True,
+                    force: bool = False) -> str:
     import torch
     from torch.utils import cpp_extension as ce
 
-    srcs = [os.path.join(CSRC, s) for s in SOURCES]
-    hdrs = [os.path.join(CSRC, "common.h")]
+    mod_name, sources, headers = EXTENSIONS[ext]
+    SO_PATH = extension_path(ext)
+    srcs = [os.path.join(CSRC, s) for s in sources]
+    hdrs = [os.path.join(CSRC, h) for h in headers]
     if not force and os.path.exists(SO_PATH):
         so_mtime = os.path.getmtime(SO_PATH)
         if all(os.path.getmtime(f) < so_mtime for f in srcs + hdrs):
             return SO_PATH
+    # build next to the target and rename: a concurrent reader never sees
+    # a half-written library
+    final_path, SO_PATH = SO_PATH, SO_PATH + ".%d.tmp" % os.getpid()
 
     hipcc = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "bin", "hipcc")
     torch_lib = ce.library_paths()[0]
@@ -50,7 +83,9 @@ def build(verbose: bool = True, force: bool = False) -> str:
         "-std=c++17",
         "-shared",
         "-fPIC",
-        "-DTORCH_EXTENSION_NAME=_C",
+        f"-DTORCH_EXTENSION_NAME={mod_name}",
+        # packed-fp32 VALU forms are kept out of generated code
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
         "-DTORCH_API_INCLUDE_EXTENSION_H",
         f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
         *getattr(ce, "COMMON_HIP_FLAGS", ["-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1"]),
@@ -72,10 +107,15 @@ def build(verbose: bool = True, force: bool = False) -> str:
     ]
     if verbose:
         print("[fusioninfer build]", " ".join(cmd), file=sys.stderr)
-    subprocess.run(cmd, check=True)
-    return SO_PATH
+    subprocess.run(cmd, check=True,
+                   stdout=None if verbose else subprocess.DEVNULL,
+                   stderr=None if verbose else subprocess.DEVNULL)
+    os.replace(SO_PATH, final_path)
+    return final_path
 
 
 if __name__ == "__main__":
-    build(force="--force" in sys.argv)
-    print(SO_PATH)
+    which = [a for a in sys.argv[1:] if not a.startswith("-")] or ["all"]
+    names = list(EXTENSIONS) if "all" in which else which
+    for name in names:
+        print(build_extension(name, force="--force" in sys.argv))

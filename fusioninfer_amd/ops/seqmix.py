@@ -1,0 +1,158 @@
+"""Sequence-mixer ops: scalar-gain RMS norms on an fp32 residual stream,
+token shift, shared-key/value rotary attention with chunk/window masks
+over the paged cache, the generalized delta rule and its gated output,
+and the tanh-GELU gated MLP activation.
+
+Dispatch follows the package policy: GPU tensors run the hand-written
+CDNA4 kernels of the ``_C_seqmix`` extension (activations in bf16 or
+fp32, statistics/state always fp32) and raise if it is not built; CPU
+tensors run the PyTorch implementations in ``seqmix_reference``.
+
+The extension is separate from ``_C`` so that a model that needs only
+these ops compiles only these sources on first use.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from fusioninfer_amd.ops import seqmix_reference as ref
+
+_C = None
+_C_ERR: Optional[BaseException] = None
+
+
+def _load():
+    global _C, _C_ERR
+    if _C is not None:
+        return _C
+    try:
+        import importlib
+
+        _C = importlib.import_module("fusioninfer_amd.ops._C_seqmix")
+    except Exception as e:  # noqa: BLE001 - reported by _native()
+        _C_ERR = e
+    return _C
+
+
+def has_native() -> bool:
+    return _load() is not None
+
+
+def _native():
+    c = _load()
+    if c is None:
+        raise RuntimeError(
+            "fusioninfer_amd sequence-mixer extension (_C_seqmix.so) is not "
+            "available but a GPU tensor was passed; build it with "
+            "`python -m fusioninfer_amd.ops.build seqmix`."
+        ) from _C_ERR
+    return c
+
+
+def scalar_rms_norm(x, g, eps: float, out_dtype):
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _native().scalar_rms_norm(out, x, g, eps)
+        return out
+    return ref.scalar_rms_norm(x, g, eps, out_dtype)
+
+
+def residual_add_scalar_norm_(resid, y, g_post, eps: float, g_next=None,
+                              out_dtype=None):
+    if resid.is_cuda:
+        out = None
+        if g_next is not None:
+            out = torch.empty(resid.shape, dtype=out_dtype,
+                              device=resid.device)
+        _native().residual_add_scalar_norm(resid, y, g_post, g_next, out, eps)
+        return out
+    return ref.residual_add_scalar_norm_(resid, y, g_post, eps, g_next,
+                                         out_dtype)
+
+
+def norm_token_shift(resid, g, shift, state, seq_cu, row_seq, positions,
+                     seq_slots, eps: float, out_dtype):
+    if resid.is_cuda:
+        out = torch.empty(resid.shape, dtype=out_dtype, device=resid.device)
+        _native().norm_token_shift(out, resid, g, shift, state, seq_cu,
+                                   row_seq, positions, seq_slots, eps)
+        return out
+    return ref.norm_token_shift(resid, g, shift, state, seq_cu, row_seq,
+                                positions, seq_slots, eps, out_dtype)
+
+
+def rope_unitnorm_cache_(q, k, positions, inv_freq, eps: float, k_cache,
+                         v_cache, slot_mapping, num_heads: int,
+                         num_kv_heads: int, head_dim: int):
+    """q/k may be column slices of one projection output (row stride >
+    width); returns a fresh contiguous processed q [T, H, D]."""
+    if q.is_cuda:
+        T = q.shape[0]
+        out = torch.empty((T, num_heads, head_dim), dtype=q.dtype,
+                          device=q.device)
+        _native().rope_unitnorm_cache(out, q, k, positions, inv_freq,
+                                      k_cache, v_cache, slot_mapping,
+                                      num_heads, num_kv_heads, head_dim, eps)
+        return out
+    return ref.rope_unitnorm_cache_(q, k, positions, inv_freq, eps, k_cache,
+                                    v_cache, slot_mapping, num_heads,
+                                    num_kv_heads, head_dim)
+
+
+def ranged_paged_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
+                           scale: float, chunk: int = 0, window: int = 0,
+                           seq_cu=None, max_rows: int = 0):
+    """``seq_cu``/``max_rows`` (longest row group of the step) let the GPU
+    path pick the tiled MFMA kernel for multi-row groups; without them
+    (or for one-row groups) the row-per-wave kernel runs."""
+    if q.is_cuda:
+        T, H, D = q.shape
+        out = torch.empty((T, H, v_cache.shape[3]), dtype=q.dtype,
+                          device=q.device)
+        _native().ranged_paged_attention(out, q, k_cache, v_cache, seq_bt,
+                                         row_seq, positions, scale,
+                                         int(chunk), int(window))
+        return out
+    return ref.ranged_paged_attention(q, k_cache, v_cache, seq_bt, row_seq,
+                                      positions, scale, chunk, window)
+
+
+def delta_rule(r, k, v, wlin, alin, glin, w0, a_bias, norm_w, state,
+               seq_cu, seq_slots, positions, heads: int, dim: int,
+               eps: float, decay_scale: float):
+    if r.is_cuda:
+        T = r.shape[0]
+        out = torch.empty((T, heads * dim), dtype=r.dtype, device=r.device)
+        _native().delta_rule(out, r, k, v, wlin, alin, glin, w0, a_bias,
+                             norm_w, state, seq_cu, seq_slots, positions,
+                             heads, dim, eps, decay_scale)
+        return out
+    return ref.delta_rule(r, k, v, wlin, alin, glin, w0, a_bias, norm_w,
+                          state, seq_cu, seq_slots, positions, heads, dim,
+                          eps, decay_scale)
+
+
+def dual_norm_combine_residual_(resid, yl, yr, wl, wr, g_post, eps: float,
+                                g_next=None, out_dtype=None):
+    if resid.is_cuda:
+        out = None
+        if g_next is not None:
+            out = torch.empty(resid.shape, dtype=out_dtype,
+                              device=resid.device)
+        _native().dual_norm_combine_residual(resid, yl, yr, wl, wr, g_post,
+                                             g_next, out, eps)
+        return out
+    return ref.dual_norm_combine_residual_(resid, yl, yr, wl, wr, g_post,
+                                           eps, g_next, out_dtype)
+
+
+def gelu_tanh_and_mul(gu):
+    if gu.is_cuda:
+        out = torch.empty((gu.shape[0], gu.shape[1] // 2), dtype=gu.dtype,
+                          device=gu.device)
+        _native().gelu_tanh_and_mul(out, gu)
+        return out
+    return ref.gelu_tanh_and_mul(gu)

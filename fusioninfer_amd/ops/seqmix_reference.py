@@ -1,0 +1,208 @@
+"""PyTorch implementations of the sequence-mixer ops (ops/seqmix.py).
+
+These are the CPU execution path and the numerics oracle the HIP kernels
+of ``_C_seqmix`` are tested against. Everything that the kernels keep in
+32-bit (norm statistics, residual stream, rotary angles, attention scores
+and softmax, decays, gates and the recurrent state) is fp32 here as well;
+``out_dtype`` only rounds what is handed to the next matrix product.
+
+Batch layout shared by all ops: the step's token rows are grouped by
+sequence, ``seq_cu[s]:seq_cu[s+1]`` are the rows of sequence ``s`` (a
+decoding sequence is a one-row group), ``row_seq[t]`` is the group of row
+``t``, ``positions[t]`` its absolute position, ``seq_slots[s]`` the
+sequence's state slot (-1: no state kept) and ``seq_bt[s]`` its block
+table into the paged cache.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+
+def _rms(x: torch.Tensor, eps: float) -> torch.Tensor:
+    return x * torch.rsqrt(x.pow(2).mean(dim=-1, keepdim=True) + eps)
+
+
+def scalar_rms_norm(x, g, eps: float, out_dtype):
+    """x / sqrt(mean(x^2) + eps) * g with ONE gain for all coordinates."""
+    return (_rms(x.float(), eps) * g.float()).to(out_dtype)
+
+
+def residual_add_scalar_norm_(resid, y, g_post, eps: float, g_next=None,
+                              out_dtype=None):
+    """resid += rms(y) * g_post (fp32, in place); optionally returns the
+    next sublayer's input rms(resid) * g_next."""
+    resid.add_(_rms(y.float(), eps) * g_post.float())
+    if g_next is None:
+        return None
+    return (_rms(resid, eps) * g_next.float()).to(out_dtype)
+
+
+def norm_token_shift(resid, g, shift, state, seq_cu, row_seq, positions,
+                     seq_slots, eps: float, out_dtype):
+    """h = rms(resid) * g, then every row is pulled towards the previous
+    token's h: h + (h_prev - h) * shift. The previous token of a group's
+    first row comes from ``state`` (zeros at position 0); the group's last
+    h is stored back."""
+    h = _rms(resid, eps) * g.float()
+    prev = torch.zeros_like(h)
+    prev[1:] = h[:-1]
+    cu = seq_cu.tolist()
+    slots = seq_slots.tolist()
+    pos = positions.tolist()
+    for s in range(len(slots)):
+        a, b = cu[s], cu[s + 1]
+        if b <= a:
+            continue
+        if pos[a] == 0 or slots[s] < 0:
+            prev[a] = 0
+        else:
+            prev[a] = state[slots[s]]
+        if slots[s] >= 0:
+            state[slots[s]] = h[b - 1]
+    return (h + (prev - h) * shift.float()).to(out_dtype)
+
+
+def rope_unitnorm_cache_(q, k, positions, inv_freq, eps: float, k_cache,
+                         v_cache, slot_mapping, num_heads: int,
+                         num_kv_heads: int, head_dim: int):
+    """Interleaved-pair rotary embedding on the first 2*len(inv_freq)
+    dims of every q/k head, then each head divided by its RMS (no gain).
+    The UNPROCESSED k rows go to ``v_cache`` (shared key/value projection),
+    the processed ones to ``k_cache``. Returns processed q [T, H, D]."""
+    T = q.shape[0]
+    qf = q.float().reshape(T, num_heads, head_dim)
+    kf = k.float().reshape(T, num_kv_heads, head_dim)
+    ang = positions.float()[:, None] * inv_freq.float()[None, :]
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    rd = 2 * inv_freq.numel()
+
+    def rot(t):
+        t = t.clone()
+        u, w = t[..., 0:rd:2].clone(), t[..., 1:rd:2].clone()
+        t[..., 0:rd:2] = u * c - w * s
+        t[..., 1:rd:2] = w * c + u * s
+        return t
+
+    qo = _rms(rot(qf), eps)
+    ko = _rms(rot(kf), eps)
+    bs = k_cache.shape[2]
+    slots = slot_mapping.long()
+    ok = slots >= 0
+    blk, off = slots[ok] // bs, slots[ok] % bs
+    k_cache[blk, :, off, :] = ko[ok].to(k_cache.dtype)
+    v_cache[blk, :, off, :] = kf[ok].to(v_cache.dtype)
+    return qo.to(q.dtype)
+
+
+def ranged_paged_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
+                           scale: float, chunk: int = 0, window: int = 0):
+    """Softmax attention of every row over the paged keys of its own
+    sequence at positions lo..p, where p is the row's position and lo is
+    the start of p's chunk (``chunk`` > 0: chunks of that many positions
+    counted from 0) and/or p - window + 1 (``window`` > 0)."""
+    T, H, D = q.shape
+    G, bs = k_cache.shape[1], k_cache.shape[2]
+    rep = H // G
+    out = torch.zeros(T, H, v_cache.shape[3], dtype=torch.float32)
+    pos = positions.tolist()
+    rs = row_seq.tolist()
+    qf = q.float()
+    t = 0
+    while t < T:
+        # rows of one sequence that share a key range start are batched
+        s = rs[t]
+        e = t
+        while e + 1 < T and rs[e + 1] == s:
+            e += 1
+        p0, p1 = pos[t], pos[e]
+        lo_all = 0
+        if chunk > 0:
+            lo_all = (p0 // chunk) * chunk
+        if window > 0:
+            lo_all = max(lo_all, p0 - window + 1)
+        idx = torch.arange(lo_all, p1 + 1)
+        blocks = seq_bt[s].long()[idx // bs]
+        kk = k_cache[blocks, :, idx % bs, :].float()   # [L, G, D]
+        vv = v_cache[blocks, :, idx % bs, :].float()
+        kk = kk.repeat_interleave(rep, dim=1)
+        vv = vv.repeat_interleave(rep, dim=1)
+        pr = torch.tensor(pos[t:e + 1])
+        sc = torch.einsum("ihd,jhd->hij", qf[t:e + 1], kk) * scale
+        vis = idx[None, :] <= pr[:, None]
+        if chunk > 0:
+            vis &= (idx[None, :] // chunk) == (pr[:, None] // chunk)
+        if window > 0:
+            vis &= idx[None, :] > (pr[:, None] - window)
+        sc = sc.masked_fill(~vis[None], float("-inf"))
+        w = torch.softmax(sc, dim=-1)
+        out[t:e + 1] = torch.einsum("hij,jhd->ihd", w, vv)
+        t = e + 1
+    return out.to(q.dtype)
+
+
+def delta_rule(r, k, v, wlin, alin, glin, w0, a_bias, norm_w, state,
+               seq_cu, seq_slots, positions, heads: int, dim: int,
+               eps: float, decay_scale: float):
+    """Generalized delta rule with per-channel decay and removal rate.
+
+    Per head, with u = k / sqrt(|k|^2 + 1e-6),
+    w = exp(-decay_scale * sigmoid(wlin + w0)), a = sigmoid(alin + a_bias):
+        S <- diag(w) S - (a*u) (u^T S) + k v^T      (both terms read old S)
+        o  = S^T r
+    o is divided by its RMS per head, scaled by norm_w and sigmoid(glin).
+    ``state`` [slots, heads, dim, dim] fp32 carries S between steps (zero
+    at position 0)."""
+    T = r.shape[0]
+    rf = r.float().reshape(T, heads, dim)
+    kf = k.float().reshape(T, heads, dim)
+    vf = v.float().reshape(T, heads, dim)
+    w = torch.exp(-decay_scale * torch.sigmoid(wlin.float() + w0.float()))
+    w = w.reshape(T, heads, dim)
+    a = torch.sigmoid(alin.float() + a_bias.float()).reshape(T, heads, dim)
+    u = kf * torch.rsqrt(kf.pow(2).sum(dim=-1, keepdim=True) + 1e-6)
+    au = a * u
+    o = torch.empty(T, heads, dim, dtype=torch.float32)
+    cu = seq_cu.tolist()
+    slots = seq_slots.tolist()
+    pos = positions.tolist()
+    for s in range(len(slots)):
+        a0, b0 = cu[s], cu[s + 1]
+        if b0 <= a0:
+            continue
+        if pos[a0] == 0 or slots[s] < 0:
+            S = torch.zeros(heads, dim, dim, dtype=torch.float32)
+        else:
+            S = state[slots[s]].clone()
+        for t in range(a0, b0):
+            uS = torch.einsum("hi,hij->hj", u[t], S)
+            S = (w[t][:, :, None] * S - au[t][:, :, None] * uS[:, None, :]
+                 + kf[t][:, :, None] * vf[t][:, None, :])
+            o[t] = torch.einsum("hij,hi->hj", S, rf[t])
+        if slots[s] >= 0:
+            state[slots[s]] = S
+    o = _rms(o, eps).reshape(T, heads * dim)
+    o = o * norm_w.float() * torch.sigmoid(glin.float())
+    return o.to(r.dtype)
+
+
+def dual_norm_combine_residual_(resid, yl, yr, wl, wr, g_post, eps: float,
+                                g_next=None, out_dtype=None):
+    """y = (rms(yl) * wl + rms(yr) * wr) / 2; resid += rms(y) * g_post;
+    optionally returns rms(resid) * g_next."""
+    y = 0.5 * (_rms(yl.float(), eps) * wl.float()
+               + _rms(yr.float(), eps) * wr.float())
+    resid.add_(_rms(y, eps) * g_post.float())
+    if g_next is None:
+        return None
+    return (_rms(resid, eps) * g_next.float()).to(out_dtype)
+
+
+def gelu_tanh_and_mul(gu):
+    """gu: [T, 2F] (gate | up) -> gelu_tanh(gate) * up."""
+    g, u = gu.float().chunk(2, dim=-1)
+    act = 0.5 * g * (1.0 + torch.tanh(
+        math.sqrt(2.0 / math.pi) * (g + 0.044715 * g * g * g)))
+    return (act * u).to(gu.dtype)
