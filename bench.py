@@ -70,7 +70,146 @@ def parse_args():
                         "length, and make prompts locally repetitive so the "
                         "prompt-lookup proposer has matches (spec-decode "
                         "workload mode; headline stays spec-off)")
+    p.add_argument("--mixer-compare", action="store_true",
+                   help="instead of the serving benchmark: prefill and "
+                        "decode token throughput of the Pinuvik design at "
+                        "real-model layer sizes (random weights) next to "
+                        "the Qwen3-style transformer of the same sizes")
+    p.add_argument("--mc-sizes", default="2048x16,4096x32",
+                   help="WIDTHxHEADS list for --mixer-compare (head dim "
+                        "128, kv heads = heads/4, ff = 3*width)")
+    p.add_argument("--mc-archs", default="pinuvik,transformer")
+    p.add_argument("--mc-layers", type=int, default=4)
+    p.add_argument("--mc-prompt", type=int, default=2048)
+    p.add_argument("--mc-prefill-seqs", type=int, default=4)
+    p.add_argument("--mc-decode-batch", type=int, default=64)
+    p.add_argument("--mc-chunk", type=int, default=1024,
+                   help="attention chunk (mask size) of the Pinuvik layers")
     return p.parse_args()
+
+
+def _mixer_compare_config(arch, width, heads, layers, chunk, vocab=32000):
+    from fusioninfer_amd.models.registry import (
+        get_model_config,
+        model_config_from_dict,
+    )
+
+    kv, dim, ff = max(heads // 4, 1), 128, 3 * width
+    if arch == "transformer":
+        mc = get_model_config("Qwen3-8B")
+        mc.name = f"qwen3-style-{width}x{heads}"
+        mc.hidden_size, mc.num_layers = width, layers
+        mc.num_heads, mc.num_kv_heads, mc.head_dim = heads, kv, dim
+        mc.intermediate_size, mc.vocab_size = ff, vocab
+        return mc
+    layer = {
+        "type": "parallel",
+        "mixer": {
+            "left": {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim,
+                     "scale": dim ** -0.5, "mask": {"size": chunk},
+                     "rot": {"dims": dim, "base": 1e6}},
+            # the recurrent half at half the attention's head count
+            "right": {"heads": max(heads // 2, 1), "dim": dim,
+                      "decay_rank": 64},
+        },
+        "mlp": {"kind": "dense", "ff": ff},
+    }
+    raw = {"architecture": "Pinuvik", "vocab": vocab, "width": width,
+           "norm": {"eps": 1e-5}, "layers": [layer] * layers,
+           "loop": {"start": 0, "stop": 0, "times": 1}}
+    mc = model_config_from_dict(raw)
+    mc.name = f"pinuvik-{width}x{heads}"
+    return mc
+
+
+def run_mixer_compare(args):
+    """Prefill: --mc-prefill-seqs prompts of --mc-prompt tokens as ONE
+    engine step (forced_step: the engine's own batch path without
+    sampling). Decode: --mc-decode-batch sequences at that context, one
+    token each per step (hipGraph replay). Tokens/s per arch and size."""
+    from fusioninfer_amd.config import (
+        CacheConfig,
+        EngineConfig,
+        SchedulerConfig,
+    )
+    from fusioninfer_amd.engine.llm_engine import LLMEngine
+
+    use_cuda = torch.cuda.is_available()
+    device = "cuda:0" if use_cuda else "cpu"
+    P, NS, B = args.mc_prompt, args.mc_prefill_seqs, args.mc_decode_batch
+    rows = []
+    for size in args.mc_sizes.split(","):
+        width, heads = (int(x) for x in size.lower().split("x"))
+        for arch in args.mc_archs.split(","):
+            mc = _mixer_compare_config(arch, width, heads, args.mc_layers,
+                                       args.mc_chunk)
+            tokens_cap = B * (P + 64 + args.steps + args.warmup) + NS * P
+            cfg = EngineConfig(
+                model=mc,
+                cache=CacheConfig(num_gpu_blocks=tokens_cap // 16 + B + NS,
+                                  enable_prefix_caching=False),
+                scheduler=SchedulerConfig(
+                    max_num_seqs=B, max_num_batched_tokens=max(NS * P, B * P),
+                    max_model_len=P + 64 + args.steps + args.warmup + 16),
+                enforce_eager=args.enforce_eager, seed=7,
+                num_state_slots=B + NS,
+            )
+            engine = LLMEngine(cfg, device=device)
+            if hasattr(engine.runner.model, "randomize_small_params"):
+                engine.runner.model.randomize_small_params(1)
+            gen = torch.Generator().manual_seed(5)
+            prompt = lambda: torch.randint(
+                0, mc.vocab_size, (P,), generator=gen).tolist()
+            sync = torch.cuda.synchronize if use_cuda else (lambda: None)
+
+            def prefill_once(tag):
+                ids = [f"{tag}-{i}" for i in range(NS)]
+                engine.forced_step([(i, prompt(), [P - 1]) for i in ids], ids)
+
+            for w in range(max(args.warmup // 4, 2)):
+                prefill_once(f"w{w}")
+            sync()
+            n_pf = max(args.steps // 8, 3)
+            t0 = time.monotonic()
+            for w in range(n_pf):
+                prefill_once(f"p{w}")
+            sync()
+            pf_s = (time.monotonic() - t0) / n_pf
+            # decode: admit B contexts (in groups so that one step's
+            # activations stay modest), then one token each per step
+            ids = [f"d{i}" for i in range(B)]
+            for a in range(0, B, NS):
+                engine.forced_step(
+                    [(i, prompt(), []) for i in ids[a:a + NS]])
+            step = lambda: engine.forced_step([(i, [1], [0]) for i in ids])
+            for _ in range(args.warmup):
+                step()
+            sync()
+            t0 = time.monotonic()
+            for _ in range(args.steps):
+                step()
+            sync()
+            dec_s = (time.monotonic() - t0) / args.steps
+            engine.forced_step([], ids)
+            rows.append({
+                "arch": arch, "width": width, "heads": heads,
+                "layers": args.mc_layers,
+                "prefill_tokens_per_s": round(NS * P / pf_s, 1),
+                "prefill_ms": round(pf_s * 1e3, 3),
+                "decode_tokens_per_s": round(B / dec_s, 1),
+                "decode_ms_per_step": round(dec_s * 1e3, 3),
+            })
+            del engine
+            if use_cuda:
+                torch.cuda.empty_cache()
+    print(json.dumps({
+        "metric": "mixer-compare tokens/s (prefill, decode)",
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "dtype": "bf16", "data": "synthetic",
+        "config": {"prompt_len": P, "prefill_seqs": NS, "decode_batch": B,
+                   "chunk": args.mc_chunk},
+        "rows": rows,
+    }))
 
 
 class ClosedLoopLoad:
@@ -144,6 +283,8 @@ class ClosedLoopLoad:
 
 def main():
     args = parse_args()
+    if args.mixer_compare:
+        return run_mixer_compare(args)
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))
     local_rank = int(os.environ.get("LOCAL_RANK", "0"))

@@ -479,3 +479,32 @@ def test_state_slot_manager_and_scheduler_limits():
     assert a.state_slot == -1 and sm.allocate(c) == 0
     sm.free(a)  # freeing twice is a no-op
     assert sm.num_free() == 0
+
+
+@pytest.mark.gpu
+def test_hipgraph_decode_replays_match_oracle():
+    """All-decode steps replay captured graphs (batch buckets 1, 2, 4);
+    replays alternate with eager prefill portions and with steps of other
+    batch sizes, and every replay is compared with the oracle."""
+    raw = small_config()
+    eng, W = make_engine(raw, "cuda", eager=False, blocks=48)
+    assert eng.runner._graphs, "decode graphs were not captured"
+    reqs = {k: tokens(n, s) for k, n, s in
+            [("a", 30, 1), ("b", 26, 2), ("c", 22, 3)]}
+    ref = {k: oracle.forward(raw, W, v) for k, v in reqs.items()}
+    t = reqs
+    steps = [[("a", t["a"][:8], list(range(8)))],
+             [("b", t["b"][:5], list(range(5))), ("a", t["a"][8:9], [0])]]
+    for i in range(9, 20):          # graph replays, batch 2
+        steps.append([("a", t["a"][i:i + 1], [0]),
+                      ("b", t["b"][i - 4:i - 3], [0])])
+    steps.append([("c", t["c"][:12], list(range(12)))])   # eager between
+    for i in range(20, 30):         # graph replays, batch 3 -> bucket 4
+        steps.append([("a", t["a"][i:i + 1], [0]),
+                      ("b", t["b"][i - 4:i - 3], [0]),
+                      ("c", t["c"][i - 8:i - 7], [0])])
+    got = run_schedule(eng, steps)
+    for k in reqs:
+        ps = sorted(got[k])
+        rows = torch.stack([got[k][p] for p in ps])
+        assert rel_err(rows, ref[k][ps]) < TOL, k
