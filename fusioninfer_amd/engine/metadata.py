@@ -35,6 +35,9 @@ class AttnMetadata:
     seq_bt: Optional[torch.Tensor] = None        # [S, max_blocks] int32
     seq_slots: Optional[torch.Tensor] = None     # [S] int32 state slot (-1 none)
     max_seq_rows: int = 0                        # longest group (host int)
+    # tile table over the prefill groups for tiled sequence-mixer kernels
+    # (ops.seqmix.build_attention_tiles); None on all-decode steps
+    seq_tiles: Optional[tuple] = None
     # LoRA groups for this step (fusioninfer_amd.lora.LoRABatch) or None
     lora: object = None
 

@@ -244,6 +244,11 @@ class ModelRunner:
         meta.seq_bt = torch.from_numpy(bt_np).to(dev)
         meta.seq_slots = torch.tensor(slots, dtype=torch.int32, device=dev)
         meta.max_seq_rows = max(lens, default=0)
+        if prefill_payload is not None and prefill_payload["new_lens"]:
+            from fusioninfer_amd.ops import seqmix
+
+            meta.seq_tiles = seqmix.build_attention_tiles(
+                prefill_payload["new_lens"], device=dev)
         return meta
 
     def _lora_batch(self, prefill_payload, decode_payload, np_=0):

@@ -115,7 +115,7 @@ class SharedKVAttention(nn.Module):
         o = seqmix.ranged_paged_attention(
             qn, k_cache, v_cache, meta.seq_bt, meta.row_seq, meta.positions,
             c.scale, chunk=c.chunk, window=c.window, seq_cu=meta.seq_cu,
-            max_rows=meta.max_seq_rows)
+            tiles=meta.seq_tiles)
         return self.o_proj(o.view(o.shape[0], c.heads * c.vdim))
 
 

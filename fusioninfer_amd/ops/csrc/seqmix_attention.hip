@@ -9,7 +9,17 @@
 //    lo from the chunk and/or window mask — 64 keys per step with an
 //    online fp32 softmax. One-row (decode) groups and short rows use it.
 //
+//  * ranged_paged_attention (tiled MFMA form): a 4-wave workgroup takes
+//    64 consecutive rows of one (sequence, head) and walks the key range
+//    that any of them sees in LDS-staged tiles; S^T = K Q^T and
+//    O^T = V^T P^T run on the matrix cores (bf16 16x16x16, or true-fp32
+//    16x16x4 for fp32 activations), softmax statistics stay fp32 per
+//    lane (one query per lane column, so no cross-lane transposes).
+//    Prompt portions use it.
+//
 // Cache layout: [num_blocks, kv_heads, block_size, head_dim].
+
+#include <type_traits>
 
 #include "seqmix.h"
 
@@ -166,6 +176,228 @@ __global__ __launch_bounds__(64 * kAttnWaves) void ranged_attention_row_kernel(
   }
 }
 
+
+typedef __attribute__((ext_vector_type(4))) short short4v;
+typedef __attribute__((ext_vector_type(4))) float floatx4;
+
+constexpr int kTileRows = 64;  // q rows per workgroup (16 per wave)
+
+template <typename A, int D, int BN>
+__global__ __launch_bounds__(256) void ranged_attention_tile_kernel(
+    A* __restrict__ out, const A* __restrict__ q,
+    const A* __restrict__ k_cache, const A* __restrict__ v_cache,
+    const int* __restrict__ seq_bt, int bt_stride,
+    const int* __restrict__ seq_cu, const int* __restrict__ positions,
+    const int* __restrict__ tile_seq, const int* __restrict__ tile_row0, int H,
+    int G, int block_size, float scale, int chunk, int window) {
+  constexpr bool BF = std::is_same<A, u16>::value;
+  constexpr int VEC = BF ? 8 : 4;               // elements per 16-byte load
+  constexpr int KP = D + (BF ? 8 : 4);          // K tile [BN][KP]
+  constexpr int VP = BF ? BN + 8 : D + 4;       // bf16: V^T [D][VP]; fp32: V [BN][VP]
+  constexpr int NB = BN / 16;
+  constexpr int DB = D / 16;
+  __shared__ __attribute__((aligned(16))) A k_lds[BN * KP];
+  __shared__ __attribute__((aligned(16))) A v_lds[BF ? D * VP : BN * VP];
+
+  const int tid = threadIdx.x;
+  const int wave = tid / 64, lane = tid % 64;
+  const int g4 = lane / 16, c16 = lane % 16;
+  const int h = blockIdx.y;
+  const int g = h / (H / G);
+  const int s = tile_seq[blockIdx.x];
+  const int row_first = seq_cu[s] + tile_row0[blockIdx.x];
+  const int nrows = min(kTileRows, seq_cu[s + 1] - row_first);
+  const int* bt = seq_bt + static_cast<int64_t>(s) * bt_stride;
+
+  auto range_lo = [&](int p) {
+    int lo = 0;
+    if (chunk > 0) lo = (p / chunk) * chunk;
+    if (window > 0) lo = max(lo, p - window + 1);
+    return lo;
+  };
+  const int p_first = positions[row_first];
+  const int kv_lo = range_lo(p_first);
+  const int kv_hi = p_first + nrows - 1;   // positions in a group ascend by 1
+
+  // this lane's query (column c16 of the wave's 16)
+  const int my_row = wave * 16 + c16;
+  const bool row_ok = my_row < nrows;
+  const int my_pos = row_ok ? p_first + my_row : -1;
+  const int my_lo = row_ok ? range_lo(my_pos) : 0;
+  const A* qp = q + (static_cast<int64_t>(row_first + my_row) * H + h) * D;
+
+  short4v qf16[BF ? DB : 1];
+  float qf32[BF ? 1 : D / 4];
+  if constexpr (BF) {
+#pragma unroll
+    for (int kk = 0; kk < DB; ++kk) {
+      if (row_ok)
+        qf16[kk] = *reinterpret_cast<const short4v*>(qp + 16 * kk + 4 * g4);
+      else
+        qf16[kk] = short4v{0, 0, 0, 0};
+    }
+  } else {
+#pragma unroll
+    for (int kk = 0; kk < D / 4; ++kk)
+      qf32[kk] = row_ok ? qp[4 * kk + g4] : 0.f;
+  }
+
+  floatx4 o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) o[db] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  for (int j0 = kv_lo; j0 <= kv_hi; j0 += BN) {
+    // ---- stage K and V tiles (zero-filled past the range) ----
+    constexpr int VPR = D / VEC;               // vectors per key row
+    for (int vid = tid; vid < BN * VPR; vid += 256) {
+      const int key_l = vid / VPR, dv = vid % VPR;
+      const int key = j0 + key_l;
+      typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+      u32x4 kv4 = {0u, 0u, 0u, 0u}, vv4 = {0u, 0u, 0u, 0u};
+      if (key <= kv_hi) {
+        const int64_t off =
+            ((static_cast<int64_t>(bt[key / block_size]) * G + g) * block_size +
+             key % block_size) * D + dv * VEC;
+        kv4 = *reinterpret_cast<const u32x4*>(k_cache + off);
+        vv4 = *reinterpret_cast<const u32x4*>(v_cache + off);
+      }
+      *reinterpret_cast<u32x4*>(k_lds + key_l * KP + dv * VEC) = kv4;
+      if constexpr (BF) {
+        const u16* ve = reinterpret_cast<const u16*>(&vv4);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v_lds[(dv * 8 + e) * VP + key_l] = ve[e];
+      } else {
+        *reinterpret_cast<u32x4*>(v_lds + key_l * VP + dv * VEC) = vv4;
+      }
+    }
+    __syncthreads();
+
+    // ---- S^T = K Q^T, masked and scaled ----
+    float sv[NB][4];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+      const A* kr = k_lds + (nb * 16 + c16) * KP;
+      if constexpr (BF) {
+#pragma unroll
+        for (int kk = 0; kk < DB; ++kk) {
+          const short4v a =
+              *reinterpret_cast<const short4v*>(kr + 16 * kk + 4 * g4);
+          acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qf16[kk], acc, 0,
+                                                          0, 0);
+        }
+      } else {
+#pragma unroll
+        for (int kk = 0; kk < D / 4; ++kk)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[4 * kk + g4], qf32[kk],
+                                                     acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = j0 + nb * 16 + 4 * g4 + i;
+        const bool vis = key <= my_pos && key >= my_lo;
+        sv[nb][i] = vis ? acc[i] * scale : -INFINITY;
+        tmax = fmaxf(tmax, sv[nb][i]);
+      }
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m, tmax);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float corr = expf(m - m_safe);       // m = -inf -> 0
+    float psum = 0.f;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        sv[nb][i] = expf(sv[nb][i] - m_safe);  // masked -> 0
+        psum += sv[nb][i];
+      }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = m_new;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[db][i] *= corr;
+
+    // ---- O^T += V^T P^T ----
+    if constexpr (BF) {
+      short4v pf[NB];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          pf[nb][i] = static_cast<short>(f32_to_bf16(sv[nb][i]));
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const A* vr = v_lds + (db * 16 + c16) * VP;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const short4v a =
+              *reinterpret_cast<const short4v*>(vr + nb * 16 + 4 * g4);
+          o[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pf[nb], o[db],
+                                                            0, 0, 0);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            o[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                v_lds[(nb * 16 + 4 * g4 + i) * VP + db * 16 + c16], sv[nb][i],
+                o[db], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  if (!row_ok) return;
+  const float inv_l = 1.0f / l;
+  A* op = out + (static_cast<int64_t>(row_first + my_row) * H + h) * D;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      Act<A>::st(op + db * 16 + 4 * g4 + i, o[db][i] * inv_l);
+}
+
+template <typename A>
+bool launch_ranged_attention_tiles(A* out, const A* q, const A* k_cache,
+                                   const A* v_cache, const int* seq_bt,
+                                   int bt_stride, const int* seq_cu,
+                                   const int* positions, const int* tile_seq,
+                                   const int* tile_row0, int num_tiles, int H,
+                                   int G, int D, int block_size, float scale,
+                                   int chunk, int window, hipStream_t s) {
+  constexpr bool BF = std::is_same<A, u16>::value;
+  if (num_tiles == 0) return true;
+  dim3 grid(num_tiles, H);
+#define FI_TILE(DD, BNB, BNF)                                                  \
+  case DD:                                                                     \
+    hipLaunchKernelGGL(                                                        \
+        (ranged_attention_tile_kernel<A, DD, (BF ? BNB : BNF)>), grid,         \
+        dim3(256), 0, s, out, q, k_cache, v_cache, seq_bt, bt_stride, seq_cu,  \
+        positions, tile_seq, tile_row0, H, G, block_size, scale, chunk,        \
+        window);                                                               \
+    return true;
+  switch (D) {
+    FI_TILE(32, 64, 64)
+    FI_TILE(64, 64, 64)
+    FI_TILE(96, 64, 32)
+    FI_TILE(128, 64, 32)
+    FI_TILE(256, 32, 16)
+    default:
+      return false;   // caller falls back to the row-per-wave kernel
+  }
+#undef FI_TILE
+}
+
 template <typename A>
 void launch_rope_unitnorm_cache(A* q_out, const A* q, int64_t q_stride,
                                 const A* k, int64_t k_stride,
@@ -198,6 +430,10 @@ void launch_ranged_attention_rows(A* out, const A* q, const A* k_cache,
 }
 
 #define FI_INST(A)                                                             \
+  template bool launch_ranged_attention_tiles<A>(                              \
+      A*, const A*, const A*, const A*, const int*, int, const int*,           \
+      const int*, const int*, const int*, int, int, int, int, int, float, int, \
+      int, hipStream_t);                                                       \
   template void launch_rope_unitnorm_cache<A>(                                 \
       A*, const A*, int64_t, const A*, int64_t, const int*, const float*, A*,  \
       A*, const int*, int, int, int, int, int, int, float, hipStream_t);       \

@@ -38,11 +38,17 @@ void launch_ranged_attention_rows(A*, const A*, const A*, const A*, const int*,
                                   int, const int*, const int*, int, int, int,
                                   int, int, float, int, int, hipStream_t);
 template <typename A>
-void launch_delta_rule(A*, const A*, const A*, const A*, const A*, const A*,
-                       const A*, int64_t, int64_t, int64_t, int64_t, int64_t,
-                       int64_t, const float*, const float*, const float*,
-                       float*, const int*, const int*, const int*, int, int,
-                       int, float, float, hipStream_t);
+bool launch_ranged_attention_tiles(A*, const A*, const A*, const A*,
+                                   const int*, int, const int*, const int*,
+                                   const int*, const int*, int, int, int, int,
+                                   int, float, int, int, hipStream_t);
+template <typename A>
+void launch_delta_rule(A*, float*, const A*, const A*, const A*, const A*,
+                       const A*, const A*, int64_t, int64_t, int64_t, int64_t,
+                       int64_t, int64_t, const float*, const float*,
+                       const float*, float*, const int*, const int*,
+                       const int*, int, int, int, int, float, float,
+                       hipStream_t);
 }  // namespace fi
 
 namespace {
@@ -248,10 +254,18 @@ void rope_unitnorm_cache(at::Tensor q_out, at::Tensor q, at::Tensor k,
                       (float)eps, stream()));
 }
 
+// Rows [0, tile_rows) belong to the row groups that the tile tables
+// cover (tile_seq/tile_row0: group and first row inside it of every
+// 64-row tile) and run the MFMA kernel when the head size has one; all
+// other rows run the row-per-wave kernel.
 void ranged_paged_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
                             at::Tensor v_cache, at::Tensor seq_bt,
                             at::Tensor row_seq, at::Tensor positions,
-                            double scale, int64_t chunk, int64_t window) {
+                            double scale, int64_t chunk, int64_t window,
+                            c10::optional<at::Tensor> seq_cu,
+                            c10::optional<at::Tensor> tile_seq,
+                            c10::optional<at::Tensor> tile_row0,
+                            int64_t tile_rows) {
   CHECK_ACT(q);
   CHECK_ACT(out);
   CHECK_I32(row_seq);
@@ -267,15 +281,42 @@ void ranged_paged_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
   TORCH_CHECK(G >= 1 && H % G == 0 && D <= 512);
   TORCH_CHECK(row_seq.numel() == T && positions.numel() == T);
   TORCH_CHECK(chunk >= 0 && window >= 0);
+  TORCH_CHECK(tile_rows >= 0 && tile_rows <= T);
+  int64_t done = 0;
+  if (tile_rows > 0) {
+    TORCH_CHECK(seq_cu.has_value() && tile_seq.has_value() &&
+                tile_row0.has_value());
+    CHECK_I32(*seq_cu);
+    CHECK_I32(*tile_seq);
+    CHECK_I32(*tile_row0);
+    TORCH_CHECK(tile_seq->numel() == tile_row0->numel());
+    TORCH_CHECK(seq_cu->numel() <= seq_bt.size(0) + 1);
+    // head sizes without a tiled variant (or without 16-byte rows) keep
+    // the row-per-wave kernel
+    bool ok = false;
+    if ((D * k_cache.element_size()) % 16 == 0) {
+      DISPATCH_ACT(q, ok = fi::launch_ranged_attention_tiles<A>(
+                        ptr<A>(out), ptr<A>(q), ptr<A>(k_cache),
+                        ptr<A>(v_cache), seq_bt.data_ptr<int>(),
+                        (int)seq_bt.stride(0), seq_cu->data_ptr<int>(),
+                        positions.data_ptr<int>(), tile_seq->data_ptr<int>(),
+                        tile_row0->data_ptr<int>(), (int)tile_seq->numel(), H,
+                        G, D, (int)k_cache.size(2), (float)scale, (int)chunk,
+                        (int)window, stream()));
+    }
+    if (ok) done = tile_rows;
+  }
+  const int rest = T - (int)done;
   DISPATCH_ACT(q, fi::launch_ranged_attention_rows<A>(
-                      ptr<A>(out), ptr<A>(q), ptr<A>(k_cache), ptr<A>(v_cache),
-                      seq_bt.data_ptr<int>(), (int)seq_bt.stride(0),
-                      row_seq.data_ptr<int>(), positions.data_ptr<int>(), T, H,
-                      G, D, (int)k_cache.size(2), (float)scale, (int)chunk,
+                      ptr<A>(out) + done * H * D, ptr<A>(q) + done * H * D,
+                      ptr<A>(k_cache), ptr<A>(v_cache), seq_bt.data_ptr<int>(),
+                      (int)seq_bt.stride(0), row_seq.data_ptr<int>() + done,
+                      positions.data_ptr<int>() + done, rest, H, G, D,
+                      (int)k_cache.size(2), (float)scale, (int)chunk,
                       (int)window, stream()));
 }
 
-void delta_rule(at::Tensor out, at::Tensor r, at::Tensor k, at::Tensor v,
+void delta_rule(at::Tensor out, at::Tensor o_raw, at::Tensor r, at::Tensor k, at::Tensor v,
                 at::Tensor wlin, at::Tensor alin, at::Tensor glin,
                 at::Tensor w0, at::Tensor a_bias, at::Tensor norm_w,
                 at::Tensor state, at::Tensor seq_cu, at::Tensor seq_slots,
@@ -289,6 +330,8 @@ void delta_rule(at::Tensor out, at::Tensor r, at::Tensor k, at::Tensor v,
   }
   TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == T &&
               out.size(1) == n);
+  CHECK_F32(o_raw);
+  TORCH_CHECK(o_raw.numel() == T * n);
   CHECK_F32(w0);
   CHECK_F32(a_bias);
   CHECK_F32(norm_w);
@@ -300,14 +343,15 @@ void delta_rule(at::Tensor out, at::Tensor r, at::Tensor k, at::Tensor v,
   check_groups(seq_cu, seq_slots, positions, T);
   const int S = seq_slots.numel();
   DISPATCH_ACT(out, fi::launch_delta_rule<A>(
-                        ptr<A>(out), ptr<A>(r), ptr<A>(k), ptr<A>(v),
+                        ptr<A>(out), o_raw.data_ptr<float>(), ptr<A>(r),
+                        ptr<A>(k), ptr<A>(v),
                         ptr<A>(wlin), ptr<A>(alin), ptr<A>(glin), r.stride(0),
                         k.stride(0), v.stride(0), wlin.stride(0),
                         alin.stride(0), glin.stride(0), w0.data_ptr<float>(),
                         a_bias.data_ptr<float>(), norm_w.data_ptr<float>(),
                         state.data_ptr<float>(), seq_cu.data_ptr<int>(),
                         seq_slots.data_ptr<int>(), positions.data_ptr<int>(),
-                        S, (int)heads, (int)dim, (float)eps,
+                        (int)T, S, (int)heads, (int)dim, (float)eps,
                         (float)decay_scale, stream()));
 }
 

@@ -102,19 +102,41 @@ def rope_unitnorm_cache_(q, k, positions, inv_freq, eps: float, k_cache,
                                     num_kv_heads, head_dim)
 
 
+ATTENTION_TILE_ROWS = 64  # q rows per workgroup of the tiled kernel
+
+
+def build_attention_tiles(group_lens, device=None):
+    """Tile table of the tiled attention kernel: one entry per
+    ATTENTION_TILE_ROWS rows of every row group, (group, first row inside
+    the group). Returns (tile_seq, tile_row0, rows covered)."""
+    tile_seq, tile_row0 = [], []
+    for s, n in enumerate(group_lens):
+        for r0 in range(0, n, ATTENTION_TILE_ROWS):
+            tile_seq.append(s)
+            tile_row0.append(r0)
+    return (torch.tensor(tile_seq, dtype=torch.int32, device=device),
+            torch.tensor(tile_row0, dtype=torch.int32, device=device),
+            int(sum(group_lens)))
+
+
 def ranged_paged_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
                            scale: float, chunk: int = 0, window: int = 0,
-                           seq_cu=None, max_rows: int = 0):
-    """``seq_cu``/``max_rows`` (longest row group of the step) let the GPU
-    path pick the tiled MFMA kernel for multi-row groups; without them
-    (or for one-row groups) the row-per-wave kernel runs."""
+                           seq_cu=None, tiles=None):
+    """``tiles`` = build_attention_tiles(lens of the LEADING row groups):
+    on the GPU those rows run the tiled MFMA kernel (prompt portions), the
+    remaining rows (one-row decode groups) the row-per-wave kernel."""
     if q.is_cuda:
         T, H, D = q.shape
         out = torch.empty((T, H, v_cache.shape[3]), dtype=q.dtype,
                           device=q.device)
+        tile_seq = tile_row0 = None
+        tile_rows = 0
+        if tiles is not None and seq_cu is not None and tiles[2] > 0:
+            tile_seq, tile_row0, tile_rows = tiles
         _native().ranged_paged_attention(out, q, k_cache, v_cache, seq_bt,
                                          row_seq, positions, scale,
-                                         int(chunk), int(window))
+                                         int(chunk), int(window), seq_cu,
+                                         tile_seq, tile_row0, int(tile_rows))
         return out
     return ref.ranged_paged_attention(q, k_cache, v_cache, seq_bt, row_seq,
                                       positions, scale, chunk, window)
@@ -126,7 +148,9 @@ def delta_rule(r, k, v, wlin, alin, glin, w0, a_bias, norm_w, state,
     if r.is_cuda:
         T = r.shape[0]
         out = torch.empty((T, heads * dim), dtype=r.dtype, device=r.device)
-        _native().delta_rule(out, r, k, v, wlin, alin, glin, w0, a_bias,
+        o_raw = torch.empty((T, heads * dim), dtype=torch.float32,
+                            device=r.device)
+        _native().delta_rule(out, o_raw, r, k, v, wlin, alin, glin, w0, a_bias,
                              norm_w, state, seq_cu, seq_slots, positions,
                              heads, dim, eps, decay_scale)
         return out

@@ -200,7 +200,8 @@ def _attention_case(device, dim, rot, chunk, T, H=2, G=1, pos0=0, seed=0,
                                          kc, vc, mk(slots), H, G, dim)
         outs.append(seqmix.ranged_paged_attention(
             qn.view(b - a, H, dim), kc, vc, bt, mk([0] * (b - a)), mk(pos),
-            0.4, chunk=chunk, seq_cu=mk([0, b - a]), max_rows=b - a))
+            0.4, chunk=chunk, seq_cu=mk([0, b - a]),
+            tiles=seqmix.build_attention_tiles([b - a], device=device)))
     got = torch.cat(outs).reshape(T, H * dim).cpu().double()
     return got, want
 

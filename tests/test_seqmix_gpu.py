@@ -121,12 +121,14 @@ def _fill_cache(dtype, lens_total, G, D, bs, dev, seed):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,D,rot", [(4, 2, 64, 64), (3, 3, 80, 32),
-                                       (8, 1, 128, 0), (2, 2, 30, 30)])
+                                       (8, 1, 128, 0), (2, 2, 30, 30),
+                                       (2, 1, 96, 40), (2, 2, 32, 32),
+                                       (1, 1, 256, 64)])
 def test_rope_unitnorm_cache_and_attention(dtype, H, G, D, rot):
     torch.manual_seed(2)
     dev = "cuda"
     bs = 16
-    lens, pos0 = [40, 1, 9, 1], [0, 130, 57, 0]
+    lens, pos0 = [140, 1, 9, 1], [0, 130, 57, 0]
     total = [p + n for p, n in zip(pos0, lens)]
     kc, vc, bt = _fill_cache(dtype, total, G, D, bs, dev, 3)
     # earlier context of every sequence: random processed/raw keys
@@ -155,14 +157,20 @@ def test_rope_unitnorm_cache_and_attention(dtype, H, G, D, rot):
                                **tol(dtype))
     torch.testing.assert_close(kc.cpu().float(), kc2.float(), **tol(dtype))
     assert torch.equal(vc.cpu(), vc2)
+    all_tiles = seqmix.build_attention_tiles(lens, device=dev)
+    lead_tiles = seqmix.build_attention_tiles(lens[:1], device=dev)
     for chunk, window in [(0, 0), (50, 0), (0, 33), (64, 20)]:
-        o1 = seqmix.ranged_paged_attention(
-            qn.view(T, H, D), kc, vc, bt, row_seq, positions, 0.2, chunk,
-            window, seq_cu=cu, max_rows=max(lens))
         o2 = ref.ranged_paged_attention(
             qn.cpu().view(T, H, D), kc.cpu(), vc.cpu(), bt.cpu(),
             row_seq.cpu(), positions.cpu(), 0.2, chunk, window)
-        torch.testing.assert_close(o1.cpu().float(), o2.float(), **tol(dtype))
+        # row-per-wave kernel; tiled kernel on every group; tiled kernel
+        # on the leading group and rows for the rest
+        for tiles in (None, all_tiles, lead_tiles):
+            o1 = seqmix.ranged_paged_attention(
+                qn.view(T, H, D), kc, vc, bt, row_seq, positions, 0.2, chunk,
+                window, seq_cu=cu, tiles=tiles)
+            torch.testing.assert_close(o1.cpu().float(), o2.float(),
+                                       **tol(dtype))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
