@@ -43,9 +43,9 @@ bool launch_ranged_attention_tiles(A*, const A*, const A*, const A*,
                                    const int*, const int*, int, int, int, int,
                                    int, float, int, int, hipStream_t);
 template <typename A>
-void launch_delta_rule(A*, float*, const A*, const A*, const A*, const A*,
-                       const A*, const A*, int64_t, int64_t, int64_t, int64_t,
-                       int64_t, int64_t, const float*, const float*,
+void launch_delta_rule(A*, float*, float*, const A*, const A*, const A*,
+                       const A*, const A*, const A*, int64_t, int64_t, int64_t,
+                       int64_t, int64_t, int64_t, const float*, const float*,
                        const float*, float*, const int*, const int*,
                        const int*, int, int, int, int, float, float,
                        hipStream_t);
@@ -316,7 +316,7 @@ void ranged_paged_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
                       (int)window, stream()));
 }
 
-void delta_rule(at::Tensor out, at::Tensor o_raw, at::Tensor r, at::Tensor k, at::Tensor v,
+void delta_rule(at::Tensor out, at::Tensor o_raw, at::Tensor vecs, at::Tensor r, at::Tensor k, at::Tensor v,
                 at::Tensor wlin, at::Tensor alin, at::Tensor glin,
                 at::Tensor w0, at::Tensor a_bias, at::Tensor norm_w,
                 at::Tensor state, at::Tensor seq_cu, at::Tensor seq_slots,
@@ -332,6 +332,12 @@ void delta_rule(at::Tensor out, at::Tensor o_raw, at::Tensor r, at::Tensor k, at
               out.size(1) == n);
   CHECK_F32(o_raw);
   TORCH_CHECK(o_raw.numel() == T * n);
+  // scratch of the state-independent per-token vectors: 5 vectors of the
+  // kernel's row capacity per (token, head)
+  CHECK_F32(vecs);
+  const int64_t cap = dim <= 64 ? 64 : (dim <= 128 ? 128 : 256);
+  TORCH_CHECK(vecs.numel() == T * heads * 5 * cap,
+              "delta rule: scratch must hold [T, heads, 5, ", cap, "]");
   CHECK_F32(w0);
   CHECK_F32(a_bias);
   CHECK_F32(norm_w);
@@ -343,7 +349,8 @@ void delta_rule(at::Tensor out, at::Tensor o_raw, at::Tensor r, at::Tensor k, at
   check_groups(seq_cu, seq_slots, positions, T);
   const int S = seq_slots.numel();
   DISPATCH_ACT(out, fi::launch_delta_rule<A>(
-                        ptr<A>(out), o_raw.data_ptr<float>(), ptr<A>(r),
+                        ptr<A>(out), o_raw.data_ptr<float>(),
+                        vecs.data_ptr<float>(), ptr<A>(r),
                         ptr<A>(k), ptr<A>(v),
                         ptr<A>(wlin), ptr<A>(alin), ptr<A>(glin), r.stride(0),
                         k.stride(0), v.stride(0), wlin.stride(0),

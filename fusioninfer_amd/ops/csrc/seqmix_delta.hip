@@ -10,45 +10,107 @@
 //   S[i][c] <- w_i S[i][c] - a_i u_i tc + k_i v_c
 //   o_c = sum_i S[i][c] r_i
 //
-// Value columns never mix, so the work is cut into (column tile, head,
-// sequence) items of 16 columns, one 64-lane wave each: lane = (column,
-// row quarter) keeps its quarter of the column in registers (DK = row
-// capacity >= dim, compile time). The per-token vectors (w, a*u, u, k, r)
-// are computed once by the wave and broadcast through LDS; the next
-// token's inputs are fetched while the current one is applied. The state
-// is read from the sequence's slot unless the group starts at position 0
-// (or has no slot) and written back at the end.
-//
-// A second kernel turns the raw o into the mixer output: per-head
-// unit-RMS, gain, sigmoid gate.
+// Three kernels:
+//  1. delta_prep: everything per token that does not depend on the state
+//     — the fp32 vectors (w, a*u, u, k, r) of every (token, head), padded
+//     to the row capacity DK — fully parallel, one wave per (token, head).
+//  2. delta_rule_wave: the recurrence. Value columns never mix, so the
+//     work is cut into (column tile, head, sequence) items, one 64-lane
+//     wave each: lane = (column, row slice) keeps its slice of the column
+//     in registers (DK = row capacity >= dim, SL = slices per column,
+//     compile time; a wave covers 64/SL columns). Slices of one column
+//     sit in adjacent lanes, so the two per-token reductions over rows
+//     are DPP lane swaps. Tokens are staged in blocks: the block's vectors
+//     go global -> registers -> LDS while the previous block is applied
+//     from LDS, so no global round trip sits on the token-to-token chain.
+//     A workgroup is a single wave: LDS ordering needs no s_barrier.
+//     The state is read from the sequence's slot unless the group starts
+//     at position 0 (or has no slot) and written back at the end.
+//  3. delta_out_gate: per-head unit-RMS of o, gain, sigmoid gate.
 
 #include "seqmix.h"
 
 namespace fi {
 
-constexpr int kColsPerWave = 16;
+template <int CTRL>
+FI_DEV float dpp_move(float x) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL,
+                                         0xF, 0xF, true));
+}
 
-template <typename A, int DK>
+// sum over the SL adjacent lanes that hold one column (SL = 4 or 8);
+// every lane of the group ends with the total
+template <int SL>
+FI_DEV float slice_sum(float x) {
+  x += dpp_move<0xB1>(x);              // quad_perm [1,0,3,2]
+  x += dpp_move<0x4E>(x);              // quad_perm [2,3,0,1]
+  if (SL == 8) x += dpp_move<0x141>(x);  // row_half_mirror: other quad
+  return x;
+}
+
+// vecs[t][head][0..4][DK] = (w, a*u, u, k, r); entries >= dim are the
+// identity (w = 1, rest 0) so padded state rows stay zero
+template <typename A>
+__global__ __launch_bounds__(256) void delta_prep_kernel(
+    float* __restrict__ vecs, const A* __restrict__ r, const A* __restrict__ k,
+    const A* __restrict__ wlin, const A* __restrict__ alin, int64_t r_stride,
+    int64_t k_stride, int64_t w_stride, int64_t a_stride,
+    const float* __restrict__ w0, const float* __restrict__ a_bias, int T,
+    int heads, int dim, int DK, float decay_scale) {
+  const int lane = threadIdx.x % 64;
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / 64;
+  if (item >= static_cast<int64_t>(T) * heads) return;
+  const int t = static_cast<int>(item / heads);
+  const int head = static_cast<int>(item % heads);
+  const int hbase = head * dim;
+  float* dst = vecs + item * 5 * DK;
+  float ksq = 0.f;
+  for (int i = lane; i < dim; i += 64) {
+    const float kk = Act<A>::ld(k + t * k_stride + hbase + i);
+    ksq += kk * kk;
+  }
+  ksq = wave_reduce_sum(ksq);
+  const float kinv = rsqrtf(ksq + 1e-6f);
+  for (int i = lane; i < DK; i += 64) {
+    float ww = 1.f, au = 0.f, uu = 0.f, kk = 0.f, rr = 0.f;
+    if (i < dim) {
+      kk = Act<A>::ld(k + t * k_stride + hbase + i);
+      rr = Act<A>::ld(r + t * r_stride + hbase + i);
+      uu = kk * kinv;
+      ww = expf(-decay_scale *
+                sigmoidf_acc(Act<A>::ld(wlin + t * w_stride + hbase + i) +
+                             w0[hbase + i]));
+      au = sigmoidf_acc(Act<A>::ld(alin + t * a_stride + hbase + i) +
+                        a_bias[hbase + i]) * uu;
+    }
+    dst[i] = ww;
+    dst[DK + i] = au;
+    dst[2 * DK + i] = uu;
+    dst[3 * DK + i] = kk;
+    dst[4 * DK + i] = rr;
+  }
+}
+
+template <typename A, int DK, int SL>
 __global__ __launch_bounds__(64) void delta_rule_wave_kernel(
     float* __restrict__ o_raw,                  // [T, heads*dim] fp32
-    const A* __restrict__ r, const A* __restrict__ k, const A* __restrict__ v,
-    const A* __restrict__ wlin, const A* __restrict__ alin, int64_t r_stride,
-    int64_t k_stride, int64_t v_stride, int64_t w_stride, int64_t a_stride,
-    const float* __restrict__ w0, const float* __restrict__ a_bias,
-    float* __restrict__ state, const int* __restrict__ seq_cu,
-    const int* __restrict__ seq_slots, const int* __restrict__ positions,
-    int heads, int dim, float decay_scale) {
-  constexpr int RS = DK / 4;       // rows per lane
-  constexpr int EPL = DK / 64;     // vector elements per lane
-  __shared__ __attribute__((aligned(16))) float sw[DK];
-  __shared__ __attribute__((aligned(16))) float sau[DK];
-  __shared__ __attribute__((aligned(16))) float su[DK];
-  __shared__ __attribute__((aligned(16))) float sk[DK];
-  __shared__ __attribute__((aligned(16))) float sr[DK];
+    const float* __restrict__ vecs,             // [T, heads, 5, DK]
+    const A* __restrict__ v, int64_t v_stride, float* __restrict__ state,
+    const int* __restrict__ seq_cu, const int* __restrict__ seq_slots,
+    const int* __restrict__ positions, int heads, int dim) {
+  constexpr int RS = DK / SL;      // rows per lane
+  constexpr int R4 = RS / 4;
+  constexpr int COLS = 64 / SL;    // columns per wave
+  constexpr int TB = 4;            // tokens per staged block
+  constexpr int TOKF4 = 5 * DK / 4;          // float4 per token
+  constexpr int LPB = TB * TOKF4 / 64;       // float4 per lane per block
+  static_assert(RS % 4 == 0 && (TB * TOKF4) % 64 == 0, "block copy shape");
+  __shared__ __attribute__((aligned(16))) float lds[TB * 5 * DK];
   const int lane = threadIdx.x;
-  const int col = lane % kColsPerWave;
-  const int slice = lane / kColsPerWave;
-  const int c = blockIdx.x * kColsPerWave + col;
+  const int col = lane / SL;
+  const int slice = lane % SL;
+  const int c = blockIdx.x * COLS + col;
   const int head = blockIdx.y;
   const int s = blockIdx.z;
   const int row0 = seq_cu[s], row1 = seq_cu[s + 1];
@@ -56,6 +118,7 @@ __global__ __launch_bounds__(64) void delta_rule_wave_kernel(
   const int slot = seq_slots[s];
   const bool col_ok = c < dim;
   const int hbase = head * dim;
+  const int64_t tok_stride = static_cast<int64_t>(heads) * 5 * DK;
 
   float S[RS];
 #pragma unroll
@@ -70,80 +133,89 @@ __global__ __launch_bounds__(64) void delta_rule_wave_kernel(
       if (i < dim) S[j] = sp[static_cast<int64_t>(i) * dim + c];
     }
   }
-  float w0e[EPL], abe[EPL];
-#pragma unroll
-  for (int e = 0; e < EPL; ++e) {
-    const int i = lane + 64 * e;
-    w0e[e] = i < dim ? w0[hbase + i] : 0.f;
-    abe[e] = i < dim ? a_bias[hbase + i] : 0.f;
-  }
 
-  // raw inputs of the token about to be applied
-  float ke[EPL], re[EPL], we[EPL], ae[EPL], vc;
-  auto fetch = [&](int t) {
+  // the NEXT block's vectors and values, in flight while the current
+  // block is applied
+  float4 nx[LPB];
+  float nv[TB];
+  auto fetch_block = [&](int tb0) {
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) {
-      const int i = lane + 64 * e;
-      const bool ok = i < dim;
-      ke[e] = ok ? Act<A>::ld(k + t * k_stride + hbase + i) : 0.f;
-      re[e] = ok ? Act<A>::ld(r + t * r_stride + hbase + i) : 0.f;
-      we[e] = ok ? Act<A>::ld(wlin + t * w_stride + hbase + i) : 0.f;
-      ae[e] = ok ? Act<A>::ld(alin + t * a_stride + hbase + i) : 0.f;
+    for (int x = 0; x < LPB; ++x) {
+      const int f = lane + 64 * x;             // float4 index in the block
+      const int tt = f / TOKF4, within = f % TOKF4;
+      const int t = min(tb0 + tt, row1 - 1);   // tail: re-read the last row
+      nx[x] = *reinterpret_cast<const float4*>(
+          vecs + t * tok_stride + static_cast<int64_t>(head) * 5 * DK +
+          within * 4);
     }
-    vc = col_ok ? Act<A>::ld(v + t * v_stride + hbase + c) : 0.f;
+#pragma unroll
+    for (int tt = 0; tt < TB; ++tt) {
+      const int t = min(tb0 + tt, row1 - 1);
+      nv[tt] = col_ok ? Act<A>::ld(v + t * v_stride + hbase + c) : 0.f;
+    }
   };
-  fetch(row0);
+  fetch_block(row0);
 
-  for (int t = row0; t < row1; ++t) {
-    float ksq = 0.f;
+  const int i0 = slice * RS;
+  for (int tb0 = row0; tb0 < row1; tb0 += TB) {
+    // one wave per workgroup: its LDS operations complete in issue
+    // order; the wave barriers keep the compiler from reordering
+    __builtin_amdgcn_wave_barrier();
+    float vb[TB];
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) ksq += ke[e] * ke[e];
-    ksq = wave_reduce_sum(ksq);
-    const float kinv = rsqrtf(ksq + 1e-6f);
-    __syncthreads();   // single-wave workgroup: previous readers are done
+    for (int x = 0; x < LPB; ++x)
+      *reinterpret_cast<float4*>(lds + (lane + 64 * x) * 4) = nx[x];
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) {
-      const int i = lane + 64 * e;
-      const bool ok = i < dim;
-      const float uu = ke[e] * kinv;
-      const float ww =
-          ok ? expf(-decay_scale * sigmoidf_acc(we[e] + w0e[e])) : 1.f;
-      const float aa = ok ? sigmoidf_acc(ae[e] + abe[e]) : 0.f;
-      sw[i] = ww;
-      sau[i] = aa * uu;
-      su[i] = uu;
-      sk[i] = ke[e];
-      sr[i] = re[e];
+    for (int tt = 0; tt < TB; ++tt) vb[tt] = nv[tt];
+    if (tb0 + TB < row1) fetch_block(tb0 + TB);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    const int nt = min(TB, row1 - tb0);
+#pragma unroll
+    for (int tt = 0; tt < TB; ++tt) {
+      if (tt < nt) {
+        const float* base = lds + tt * 5 * DK + i0;
+        float4 ww[R4], au[R4], uu[R4], kk[R4], rr[R4];
+#pragma unroll
+        for (int x = 0; x < R4; ++x) {
+          uu[x] = *reinterpret_cast<const float4*>(base + 2 * DK + 4 * x);
+          ww[x] = *reinterpret_cast<const float4*>(base + 4 * x);
+          au[x] = *reinterpret_cast<const float4*>(base + DK + 4 * x);
+          kk[x] = *reinterpret_cast<const float4*>(base + 3 * DK + 4 * x);
+          rr[x] = *reinterpret_cast<const float4*>(base + 4 * DK + 4 * x);
+        }
+        const float vcur = vb[tt];
+        float t0 = 0.f, t1 = 0.f, t2 = 0.f, t3 = 0.f;
+#pragma unroll
+        for (int x = 0; x < R4; ++x) {
+          t0 += uu[x].x * S[4 * x];
+          t1 += uu[x].y * S[4 * x + 1];
+          t2 += uu[x].z * S[4 * x + 2];
+          t3 += uu[x].w * S[4 * x + 3];
+        }
+        const float tc = slice_sum<SL>((t0 + t1) + (t2 + t3));
+        float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+#pragma unroll
+        for (int x = 0; x < R4; ++x) {
+          S[4 * x] = ww[x].x * S[4 * x] + (kk[x].x * vcur - au[x].x * tc);
+          S[4 * x + 1] =
+              ww[x].y * S[4 * x + 1] + (kk[x].y * vcur - au[x].y * tc);
+          S[4 * x + 2] =
+              ww[x].z * S[4 * x + 2] + (kk[x].z * vcur - au[x].z * tc);
+          S[4 * x + 3] =
+              ww[x].w * S[4 * x + 3] + (kk[x].w * vcur - au[x].w * tc);
+          o0 += S[4 * x] * rr[x].x;
+          o1 += S[4 * x + 1] * rr[x].y;
+          o2 += S[4 * x + 2] * rr[x].z;
+          o3 += S[4 * x + 3] * rr[x].w;
+        }
+        const float oc = slice_sum<SL>((o0 + o1) + (o2 + o3));
+        if (slice == 0 && col_ok)
+          o_raw[static_cast<int64_t>(tb0 + tt) * heads * dim + hbase + c] = oc;
+      }
     }
-    const float vcur = vc;
-    if (t + 1 < row1) fetch(t + 1);
-    __syncthreads();
-    const int i0 = slice * RS;
-    float tc = 0.f;
-#pragma unroll
-    for (int j = 0; j < RS; j += 4) {
-      const float4 uu = *reinterpret_cast<const float4*>(su + i0 + j);
-      tc += uu.x * S[j] + uu.y * S[j + 1] + uu.z * S[j + 2] + uu.w * S[j + 3];
-    }
-    tc += __shfl_xor(tc, 16, 64);
-    tc += __shfl_xor(tc, 32, 64);
-    float oc = 0.f;
-#pragma unroll
-    for (int j = 0; j < RS; j += 4) {
-      const float4 ww = *reinterpret_cast<const float4*>(sw + i0 + j);
-      const float4 au = *reinterpret_cast<const float4*>(sau + i0 + j);
-      const float4 kk = *reinterpret_cast<const float4*>(sk + i0 + j);
-      const float4 rr = *reinterpret_cast<const float4*>(sr + i0 + j);
-      S[j] = ww.x * S[j] - au.x * tc + kk.x * vcur;
-      S[j + 1] = ww.y * S[j + 1] - au.y * tc + kk.y * vcur;
-      S[j + 2] = ww.z * S[j + 2] - au.z * tc + kk.z * vcur;
-      S[j + 3] = ww.w * S[j + 3] - au.w * tc + kk.w * vcur;
-      oc += S[j] * rr.x + S[j + 1] * rr.y + S[j + 2] * rr.z + S[j + 3] * rr.w;
-    }
-    oc += __shfl_xor(oc, 16, 64);
-    oc += __shfl_xor(oc, 32, 64);
-    if (slice == 0 && col_ok)
-      o_raw[static_cast<int64_t>(t) * heads * dim + hbase + c] = oc;
   }
   if (sp != nullptr && col_ok) {
 #pragma unroll
@@ -181,9 +253,13 @@ __global__ __launch_bounds__(256) void delta_out_gate_kernel(
   }
 }
 
+inline int delta_row_capacity(int dim) {
+  return dim <= 64 ? 64 : (dim <= 128 ? 128 : 256);
+}
+
 template <typename A>
-void launch_delta_rule(A* out, float* o_raw, const A* r, const A* k,
-                       const A* v, const A* wlin, const A* alin,
+void launch_delta_rule(A* out, float* o_raw, float* vecs, const A* r,
+                       const A* k, const A* v, const A* wlin, const A* alin,
                        const A* glin, int64_t r_stride, int64_t k_stride,
                        int64_t v_stride, int64_t w_stride, int64_t a_stride,
                        int64_t g_stride, const float* w0, const float* a_bias,
@@ -192,32 +268,35 @@ void launch_delta_rule(A* out, float* o_raw, const A* r, const A* k,
                        int S, int heads, int dim, float eps, float decay_scale,
                        hipStream_t st) {
   if (S == 0 || T == 0) return;
-  dim3 grid(ceil_div(dim, kColsPerWave), heads, S);
-#define FI_LAUNCH(DK)                                                          \
-  hipLaunchKernelGGL((delta_rule_wave_kernel<A, DK>), grid, dim3(64), 0, st,   \
-                     o_raw, r, k, v, wlin, alin, r_stride, k_stride, v_stride, \
-                     w_stride, a_stride, w0, a_bias, state, seq_cu, seq_slots, \
-                     positions, heads, dim, decay_scale)
-  if (dim <= 64) {
-    FI_LAUNCH(64);
-  } else if (dim <= 128) {
-    FI_LAUNCH(128);
+  const int64_t items = static_cast<int64_t>(T) * heads;
+  const int nblk = static_cast<int>((items + 3) / 4);
+  const int DK = delta_row_capacity(dim);
+  hipLaunchKernelGGL(delta_prep_kernel<A>, dim3(nblk), dim3(256), 0, st, vecs,
+                     r, k, wlin, alin, r_stride, k_stride, w_stride, a_stride,
+                     w0, a_bias, T, heads, dim, DK, decay_scale);
+#define FI_LAUNCH(DKK, SL)                                                     \
+  hipLaunchKernelGGL((delta_rule_wave_kernel<A, DKK, SL>),                     \
+                     dim3(ceil_div(dim, 64 / SL), heads, S), dim3(64), 0, st,  \
+                     o_raw, vecs, v, v_stride, state, seq_cu, seq_slots,       \
+                     positions, heads, dim)
+  if (DK == 64) {
+    FI_LAUNCH(64, 4);
+  } else if (DK == 128) {
+    FI_LAUNCH(128, 8);
   } else {
-    FI_LAUNCH(256);
+    FI_LAUNCH(256, 8);
   }
 #undef FI_LAUNCH
-  const int64_t items = static_cast<int64_t>(T) * heads;
-  hipLaunchKernelGGL(delta_out_gate_kernel<A>,
-                     dim3(static_cast<int>((items + 3) / 4)), dim3(256), 0, st,
+  hipLaunchKernelGGL(delta_out_gate_kernel<A>, dim3(nblk), dim3(256), 0, st,
                      out, o_raw, glin, g_stride, norm_w, T, heads, dim, eps);
 }
 
 #define FI_INST(A)                                                             \
   template void launch_delta_rule<A>(                                          \
-      A*, float*, const A*, const A*, const A*, const A*, const A*, const A*,  \
-      int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, const float*,      \
-      const float*, const float*, float*, const int*, const int*, const int*,  \
-      int, int, int, int, float, float, hipStream_t);
+      A*, float*, float*, const A*, const A*, const A*, const A*, const A*,    \
+      const A*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t,          \
+      const float*, const float*, const float*, float*, const int*,            \
+      const int*, const int*, int, int, int, int, float, float, hipStream_t);
 FI_INST(float)
 FI_INST(u16)
 #undef FI_INST

@@ -150,7 +150,12 @@ def delta_rule(r, k, v, wlin, alin, glin, w0, a_bias, norm_w, state,
         out = torch.empty((T, heads * dim), dtype=r.dtype, device=r.device)
         o_raw = torch.empty((T, heads * dim), dtype=torch.float32,
                             device=r.device)
-        _native().delta_rule(out, o_raw, r, k, v, wlin, alin, glin, w0, a_bias,
+        # scratch for the state-independent per-token vectors; the last
+        # dim is the kernel's row capacity for this head size
+        cap = 64 if dim <= 64 else (128 if dim <= 128 else 256)
+        vecs = torch.empty((T, heads, 5, cap), dtype=torch.float32,
+                           device=r.device)
+        _native().delta_rule(out, o_raw, vecs, r, k, v, wlin, alin, glin, w0, a_bias,
                              norm_w, state, seq_cu, seq_slots, positions,
                              heads, dim, eps, decay_scale)
         return out

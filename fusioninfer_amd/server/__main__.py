@@ -37,6 +37,10 @@ def parse_args(argv=None):
                    help='JSON: {"kv_connector": "RcclConnector", '
                         '"kv_role": "kv_producer"|"kv_consumer"}')
     p.add_argument("--enforce-eager", action="store_true")
+    p.add_argument("--dtype", choices=["auto", "bfloat16", "float32"],
+                   default="auto",
+                   help="activation/weight dtype; float32 is available for "
+                        "families whose kernels have an fp32 path")
     p.add_argument("--quantization", choices=["fp8"], default=None)
     p.add_argument("--kv-cache-dtype", choices=["auto", "fp8"], default="auto")
     p.add_argument("--swap-space", type=float, default=0.0,
@@ -92,9 +96,16 @@ def build_engine_config(args):
             kv_rank=int(raw.get("kv_rank", 0 if role == "kv_producer" else 1)),
             kv_world_size=int(raw.get("kv_world_size", 2)),
         )
+    # --model is a registered name or a checkpoint directory whose
+    # config.json names a registered architecture (weights load from it)
     mc = get_model_config(args.model)
-    mc.model_path = args.model_path
+    if args.model_path is not None:
+        mc.model_path = args.model_path
     mc.quantization = args.quantization
+    if args.dtype != "auto":
+        if mc.architecture == "transformer" and args.dtype != "bfloat16":
+            raise SystemExit("the transformer family serves in bfloat16 only")
+        mc.dtype = args.dtype
     speculative = None
     if args.speculative_config:
         from fusioninfer_amd.engine.spec_decode import SpeculativeConfig
