@@ -16,14 +16,15 @@
 //     to the row capacity DK — fully parallel, one wave per (token, head).
 //  2. delta_rule_wave: the recurrence. Value columns never mix, so the
 //     work is cut into (column tile, head, sequence) items, one 64-lane
-//     wave each: lane = (column, row slice) keeps its slice of the column
-//     in registers (DK = row capacity >= dim, SL = slices per column,
-//     compile time; a wave covers 64/SL columns). Slices of one column
-//     sit in adjacent lanes, so the two per-token reductions over rows
-//     are DPP lane swaps. Tokens are staged in blocks: the block's vectors
-//     go global -> registers -> LDS while the previous block is applied
-//     from LDS, so no global round trip sits on the token-to-token chain.
-//     A workgroup is a single wave: LDS ordering needs no s_barrier.
+//     wave each, four waves to a workgroup: lane = (column, row slice)
+//     keeps its slice of the column in registers (DK = row capacity >=
+//     dim, SL = slices per column, compile time; a wave covers 64/SL
+//     columns). Slices of one column sit in adjacent lanes, so the two
+//     per-token reductions over rows are DPP lane swaps. Tokens are
+//     staged in blocks of TB: the block's vectors go global -> registers
+//     -> LDS (double-buffered, shared by the four waves, one barrier per
+//     block) while the previous block is applied from LDS, so no global
+//     round trip sits on the token-to-token chain.
 //     The state is read from the sequence's slot unless the group starts
 //     at position 0 (or has no slot) and written back at the end.
 //  3. delta_out_gate: per-head unit-RMS of o, gain, sigmoid gate.
@@ -39,13 +40,14 @@ FI_DEV float dpp_move(float x) {
                                          0xF, 0xF, true));
 }
 
-// sum over the SL adjacent lanes that hold one column (SL = 4 or 8);
+// sum over the SL adjacent lanes that hold one column (SL = 4, 8, 16);
 // every lane of the group ends with the total
 template <int SL>
 FI_DEV float slice_sum(float x) {
   x += dpp_move<0xB1>(x);              // quad_perm [1,0,3,2]
   x += dpp_move<0x4E>(x);              // quad_perm [2,3,0,1]
-  if (SL == 8) x += dpp_move<0x141>(x);  // row_half_mirror: other quad
+  if (SL >= 8) x += dpp_move<0x141>(x);   // row_half_mirror: other quad
+  if (SL == 16) x += dpp_move<0x140>(x);  // row_mirror: other half row
   return x;
 }
 
@@ -92,8 +94,10 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(
   }
 }
 
-template <typename A, int DK, int SL>
-__global__ __launch_bounds__(64) void delta_rule_wave_kernel(
+constexpr int kDeltaWaves = 4;   // waves (column tiles) per workgroup
+
+template <typename A, int DK, int SL, int TB>
+__global__ __launch_bounds__(64 * kDeltaWaves) void delta_rule_wave_kernel(
     float* __restrict__ o_raw,                  // [T, heads*dim] fp32
     const float* __restrict__ vecs,             // [T, heads, 5, DK]
     const A* __restrict__ v, int64_t v_stride, float* __restrict__ state,
@@ -102,15 +106,17 @@ __global__ __launch_bounds__(64) void delta_rule_wave_kernel(
   constexpr int RS = DK / SL;      // rows per lane
   constexpr int R4 = RS / 4;
   constexpr int COLS = 64 / SL;    // columns per wave
-  constexpr int TB = 4;            // tokens per staged block
-  constexpr int TOKF4 = 5 * DK / 4;          // float4 per token
-  constexpr int LPB = TB * TOKF4 / 64;       // float4 per lane per block
-  static_assert(RS % 4 == 0 && (TB * TOKF4) % 64 == 0, "block copy shape");
-  __shared__ __attribute__((aligned(16))) float lds[TB * 5 * DK];
-  const int lane = threadIdx.x;
+  constexpr int NT = 64 * kDeltaWaves;
+  constexpr int TOKF4 = 5 * DK / 4;            // float4 per token
+  constexpr int BLKF4 = TB * TOKF4;            // float4 per block
+  constexpr int LPB = (BLKF4 + NT - 1) / NT;   // float4 per thread per block
+  static_assert(RS % 4 == 0, "row slices are float4 multiples");
+  __shared__ __attribute__((aligned(16))) float lds[2][TB * 5 * DK];
+  const int tid = threadIdx.x;
+  const int lane = tid % 64;
   const int col = lane / SL;
   const int slice = lane % SL;
-  const int c = blockIdx.x * COLS + col;
+  const int c = (blockIdx.x * kDeltaWaves + tid / 64) * COLS + col;
   const int head = blockIdx.y;
   const int s = blockIdx.z;
   const int row0 = seq_cu[s], row1 = seq_cu[s + 1];
@@ -119,6 +125,7 @@ __global__ __launch_bounds__(64) void delta_rule_wave_kernel(
   const bool col_ok = c < dim;
   const int hbase = head * dim;
   const int64_t tok_stride = static_cast<int64_t>(heads) * 5 * DK;
+  const float* vhead = vecs + static_cast<int64_t>(head) * 5 * DK;
 
   float S[RS];
 #pragma unroll
@@ -141,12 +148,13 @@ __global__ __launch_bounds__(64) void delta_rule_wave_kernel(
   auto fetch_block = [&](int tb0) {
 #pragma unroll
     for (int x = 0; x < LPB; ++x) {
-      const int f = lane + 64 * x;             // float4 index in the block
-      const int tt = f / TOKF4, within = f % TOKF4;
-      const int t = min(tb0 + tt, row1 - 1);   // tail: re-read the last row
-      nx[x] = *reinterpret_cast<const float4*>(
-          vecs + t * tok_stride + static_cast<int64_t>(head) * 5 * DK +
-          within * 4);
+      const int f = tid + NT * x;              // float4 index in the block
+      if (f < BLKF4) {
+        const int tt = f / TOKF4, within = f % TOKF4;
+        const int t = min(tb0 + tt, row1 - 1);  // tail: re-read the last row
+        nx[x] = *reinterpret_cast<const float4*>(vhead + t * tok_stride +
+                                                 within * 4);
+      }
     }
 #pragma unroll
     for (int tt = 0; tt < TB; ++tt) {
@@ -157,26 +165,28 @@ __global__ __launch_bounds__(64) void delta_rule_wave_kernel(
   fetch_block(row0);
 
   const int i0 = slice * RS;
-  for (int tb0 = row0; tb0 < row1; tb0 += TB) {
-    // one wave per workgroup: its LDS operations complete in issue
-    // order; the wave barriers keep the compiler from reordering
-    __builtin_amdgcn_wave_barrier();
+  int buf = 0;
+  for (int tb0 = row0; tb0 < row1; tb0 += TB, buf ^= 1) {
+    // Buffer `buf` was last read two blocks ago; every wave has passed
+    // the barrier of the block in between since, so it is free.
     float vb[TB];
 #pragma unroll
-    for (int x = 0; x < LPB; ++x)
-      *reinterpret_cast<float4*>(lds + (lane + 64 * x) * 4) = nx[x];
+    for (int x = 0; x < LPB; ++x) {
+      const int f = tid + NT * x;
+      if (f < BLKF4) *reinterpret_cast<float4*>(&lds[buf][f * 4]) = nx[x];
+    }
 #pragma unroll
     for (int tt = 0; tt < TB; ++tt) vb[tt] = nv[tt];
+    __syncthreads();
+    // issued after the barrier (which drains outstanding loads): these
+    // have the whole apply phase to land
     if (tb0 + TB < row1) fetch_block(tb0 + TB);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
     const int nt = min(TB, row1 - tb0);
 #pragma unroll
     for (int tt = 0; tt < TB; ++tt) {
       if (tt < nt) {
-        const float* base = lds + tt * 5 * DK + i0;
+        const float* base = &lds[buf][tt * 5 * DK + i0];
         float4 ww[R4], au[R4], uu[R4], kk[R4], rr[R4];
 #pragma unroll
         for (int x = 0; x < R4; ++x) {
@@ -274,17 +284,18 @@ void launch_delta_rule(A* out, float* o_raw, float* vecs, const A* r,
   hipLaunchKernelGGL(delta_prep_kernel<A>, dim3(nblk), dim3(256), 0, st, vecs,
                      r, k, wlin, alin, r_stride, k_stride, w_stride, a_stride,
                      w0, a_bias, T, heads, dim, DK, decay_scale);
-#define FI_LAUNCH(DKK, SL)                                                     \
-  hipLaunchKernelGGL((delta_rule_wave_kernel<A, DKK, SL>),                     \
-                     dim3(ceil_div(dim, 64 / SL), heads, S), dim3(64), 0, st,  \
-                     o_raw, vecs, v, v_stride, state, seq_cu, seq_slots,       \
-                     positions, heads, dim)
+#define FI_LAUNCH(DKK, SL, TB)                                                 \
+  hipLaunchKernelGGL(                                                          \
+      (delta_rule_wave_kernel<A, DKK, SL, TB>),                                \
+      dim3(ceil_div(dim, kDeltaWaves * 64 / SL), heads, S),                    \
+      dim3(64 * kDeltaWaves), 0, st, o_raw, vecs, v, v_stride, state, seq_cu,  \
+      seq_slots, positions, heads, dim)
   if (DK == 64) {
-    FI_LAUNCH(64, 4);
+    FI_LAUNCH(64, 8, 8);
   } else if (DK == 128) {
-    FI_LAUNCH(128, 8);
+    FI_LAUNCH(128, 16, 8);
   } else {
-    FI_LAUNCH(256, 8);
+    FI_LAUNCH(256, 16, 4);
   }
 #undef FI_LAUNCH
   hipLaunchKernelGGL(delta_out_gate_kernel<A>, dim3(nblk), dim3(256), 0, st,
