@@ -164,7 +164,7 @@ def model_config_from_dict(raw: dict, model_path: Optional[str] = None,
 class PinuvikLM(nn.Module):
     """embedding -> layer runs -> scalar-gain final norm -> head.
 
-    Engine contract (same as CausalLM): ``forward(ids, meta, caches)``
+    Engine interface (same as CausalLM): ``forward(ids, meta, caches)``
     returns the final-normed hidden rows, ``compute_logits`` applies the
     head. Additionally declares per-run cache/state needs
     (``allocate_caches``/``allocate_state``) and ``uses_state_slots`` so
