@@ -10,7 +10,7 @@
 //    online fp32 softmax. One-row (decode) groups and short rows use it.
 //
 //  * ranged_paged_attention (tiled MFMA form): a 4-wave workgroup takes
-//    64 consecutive rows of one (sequence, head) and walks the key range
+//    128 consecutive rows of one (sequence, head), 32 per wave, and walks the key range
 //    that any of them sees in LDS-staged tiles; S^T = K Q^T and
 //    O^T = V^T P^T run on the matrix cores (bf16 16x16x16, or true-fp32
 //    16x16x4 for fp32 activations), softmax statistics stay fp32 per
@@ -180,7 +180,8 @@ __global__ __launch_bounds__(64 * kAttnWaves) void ranged_attention_row_kernel(
 typedef __attribute__((ext_vector_type(4))) short short4v;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
 
-constexpr int kTileRows = 64;  // q rows per workgroup (16 per wave)
+constexpr int kQSets = 2;               // 16-row query sets per wave
+constexpr int kTileRows = 64 * kQSets;  // q rows per workgroup (4 waves)
 
 template <typename A, int D, int BN>
 __global__ __launch_bounds__(256) void ranged_attention_tile_kernel(
@@ -191,6 +192,7 @@ __global__ __launch_bounds__(256) void ranged_attention_tile_kernel(
     const int* __restrict__ tile_seq, const int* __restrict__ tile_row0, int H,
     int G, int block_size, float scale, int chunk, int window) {
   constexpr bool BF = std::is_same<A, u16>::value;
+  constexpr int QS = kQSets;
   constexpr int VEC = BF ? 8 : 4;               // elements per 16-byte load
   constexpr int KP = D + (BF ? 8 : 4);          // K tile [BN][KP]
   constexpr int VP = BF ? BN + 8 : D + 4;       // bf16: V^T [D][VP]; fp32: V [BN][VP]
@@ -219,33 +221,56 @@ __global__ __launch_bounds__(256) void ranged_attention_tile_kernel(
   const int kv_lo = range_lo(p_first);
   const int kv_hi = p_first + nrows - 1;   // positions in a group ascend by 1
 
-  // this lane's query (column c16 of the wave's 16)
-  const int my_row = wave * 16 + c16;
-  const bool row_ok = my_row < nrows;
-  const int my_pos = row_ok ? p_first + my_row : -1;
-  const int my_lo = row_ok ? range_lo(my_pos) : 0;
-  const A* qp = q + (static_cast<int64_t>(row_first + my_row) * H + h) * D;
-
-  short4v qf16[BF ? DB : 1];
-  float qf32[BF ? 1 : D / 4];
-  if constexpr (BF) {
+  // this lane's queries: column c16 of each of the wave's 16-row sets
+  int my_row[QS], my_pos[QS], my_lo[QS];
+  bool row_ok[QS];
+  short4v qf16[QS][BF ? DB : 1];
+  float qf32[QS][BF ? 1 : D / 4];
 #pragma unroll
-    for (int kk = 0; kk < DB; ++kk) {
-      if (row_ok)
-        qf16[kk] = *reinterpret_cast<const short4v*>(qp + 16 * kk + 4 * g4);
-      else
-        qf16[kk] = short4v{0, 0, 0, 0};
+  for (int qs = 0; qs < QS; ++qs) {
+    my_row[qs] = (wave * QS + qs) * 16 + c16;
+    row_ok[qs] = my_row[qs] < nrows;
+    my_pos[qs] = row_ok[qs] ? p_first + my_row[qs] : -1;
+    my_lo[qs] = row_ok[qs] ? range_lo(my_pos[qs]) : 0;
+    const A* qp =
+        q + (static_cast<int64_t>(row_first + my_row[qs]) * H + h) * D;
+    if constexpr (BF) {
+#pragma unroll
+      for (int kk = 0; kk < DB; ++kk) {
+        if (row_ok[qs])
+          qf16[qs][kk] =
+              *reinterpret_cast<const short4v*>(qp + 16 * kk + 4 * g4);
+        else
+          qf16[qs][kk] = short4v{0, 0, 0, 0};
+      }
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < D / 4; ++kk)
+        qf32[qs][kk] = row_ok[qs] ? qp[4 * kk + g4] : 0.f;
     }
-  } else {
-#pragma unroll
-    for (int kk = 0; kk < D / 4; ++kk)
-      qf32[kk] = row_ok ? qp[4 * kk + g4] : 0.f;
   }
 
-  floatx4 o[DB];
+  floatx4 o[QS][DB];
+  float m[QS], l[QS];
 #pragma unroll
-  for (int db = 0; db < DB; ++db) o[db] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
+  for (int qs = 0; qs < QS; ++qs) {
+    m[qs] = -INFINITY;
+    l[qs] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) o[qs][db] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+  // bf16 activations: softmax in the log2 domain (scale * log2(e) folded
+  // into the scores, hardware exp2); fp32 activations keep expf
+  const float sc = BF ? scale * 1.4426950408889634f : scale;
+  auto ex = [](float x) {
+    return BF ? __builtin_amdgcn_exp2f(x) : expf(x);
+  };
+  // rows of this wave: 16*QS consecutive positions (the valid ones)
+  const int wave_rows = min(16 * QS, nrows - wave * 16 * QS);
+  const int wave_min_pos = wave_rows > 0 ? p_first + wave * 16 * QS : -1;
+  const int wave_max_lo =
+      wave_rows > 0 ? range_lo(p_first + wave * 16 * QS + wave_rows - 1) : 0;
+  const bool wave_full = wave_rows == 16 * QS;
 
   for (int j0 = kv_lo; j0 <= kv_hi; j0 += BN) {
     // ---- stage K and V tiles (zero-filled past the range) ----
@@ -273,65 +298,88 @@ __global__ __launch_bounds__(256) void ranged_attention_tile_kernel(
     }
     __syncthreads();
 
-    // ---- S^T = K Q^T, masked and scaled ----
-    float sv[NB][4];
-    float tmax = -INFINITY;
+    // ---- S^T = K Q^T: every K fragment read from LDS feeds QS MFMAs ----
+    // a tile every row of the wave sees completely needs no per-element
+    // mask (wave-uniform test)
+    const bool interior =
+        wave_full && j0 + BN - 1 <= wave_min_pos && j0 >= wave_max_lo;
+    float sv[QS][NB][4];
+    float tmax[QS];
+#pragma unroll
+    for (int qs = 0; qs < QS; ++qs) tmax[qs] = -INFINITY;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-      floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+      floatx4 acc[QS];
+#pragma unroll
+      for (int qs = 0; qs < QS; ++qs) acc[qs] = floatx4{0.f, 0.f, 0.f, 0.f};
       const A* kr = k_lds + (nb * 16 + c16) * KP;
       if constexpr (BF) {
 #pragma unroll
         for (int kk = 0; kk < DB; ++kk) {
           const short4v a =
               *reinterpret_cast<const short4v*>(kr + 16 * kk + 4 * g4);
-          acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qf16[kk], acc, 0,
-                                                          0, 0);
+#pragma unroll
+          for (int qs = 0; qs < QS; ++qs)
+            acc[qs] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+                a, qf16[qs][kk], acc[qs], 0, 0, 0);
         }
       } else {
 #pragma unroll
-        for (int kk = 0; kk < D / 4; ++kk)
-          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[4 * kk + g4], qf32[kk],
-                                                     acc, 0, 0, 0);
+        for (int kk = 0; kk < D / 4; ++kk) {
+          const float a = kr[4 * kk + g4];
+#pragma unroll
+          for (int qs = 0; qs < QS; ++qs)
+            acc[qs] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, qf32[qs][kk],
+                                                           acc[qs], 0, 0, 0);
+        }
       }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = j0 + nb * 16 + 4 * g4 + i;
-        const bool vis = key <= my_pos && key >= my_lo;
-        sv[nb][i] = vis ? acc[i] * scale : -INFINITY;
-        tmax = fmaxf(tmax, sv[nb][i]);
-      }
+      for (int qs = 0; qs < QS; ++qs)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = j0 + nb * 16 + 4 * g4 + i;
+          const bool vis =
+              interior || (key <= my_pos[qs] && key >= my_lo[qs]);
+          sv[qs][nb][i] = vis ? acc[qs][i] * sc : -INFINITY;
+          tmax[qs] = fmaxf(tmax[qs], sv[qs][nb][i]);
+        }
     }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(m, tmax);
-    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-    const float corr = expf(m - m_safe);       // m = -inf -> 0
-    float psum = 0.f;
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        sv[nb][i] = expf(sv[nb][i] - m_safe);  // masked -> 0
-        psum += sv[nb][i];
-      }
-    psum += __shfl_xor(psum, 16, 64);
-    psum += __shfl_xor(psum, 32, 64);
-    l = l * corr + psum;
-    m = m_new;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) o[db][i] *= corr;
-
-    // ---- O^T += V^T P^T ----
-    if constexpr (BF) {
-      short4v pf[NB];
+    for (int qs = 0; qs < QS; ++qs) {
+      float tm = tmax[qs];
+      tm = fmaxf(tm, __shfl_xor(tm, 16, 64));
+      tm = fmaxf(tm, __shfl_xor(tm, 32, 64));
+      const float m_new = fmaxf(m[qs], tm);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float corr = ex(m[qs] - m_safe);     // m = -inf -> 0
+      float psum = 0.f;
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          pf[nb][i] = static_cast<short>(f32_to_bf16(sv[nb][i]));
+        for (int i = 0; i < 4; ++i) {
+          sv[qs][nb][i] = ex(sv[qs][nb][i] - m_safe);  // masked -> 0
+          psum += sv[qs][nb][i];
+        }
+      psum += __shfl_xor(psum, 16, 64);
+      psum += __shfl_xor(psum, 32, 64);
+      l[qs] = l[qs] * corr + psum;
+      m[qs] = m_new;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[qs][db][i] *= corr;
+    }
+
+    // ---- O^T += V^T P^T: every V fragment feeds QS MFMAs ----
+    if constexpr (BF) {
+      short4v pf[QS][NB];
+#pragma unroll
+      for (int qs = 0; qs < QS; ++qs)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            pf[qs][nb][i] = static_cast<short>(f32_to_bf16(sv[qs][nb][i]));
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         const A* vr = v_lds + (db * 16 + c16) * VP;
@@ -339,8 +387,10 @@ __global__ __launch_bounds__(256) void ranged_attention_tile_kernel(
         for (int nb = 0; nb < NB; ++nb) {
           const short4v a =
               *reinterpret_cast<const short4v*>(vr + nb * 16 + 4 * g4);
-          o[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pf[nb], o[db],
-                                                            0, 0, 0);
+#pragma unroll
+          for (int qs = 0; qs < QS; ++qs)
+            o[qs][db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+                a, pf[qs][nb], o[qs][db], 0, 0, 0);
         }
       }
     } else {
@@ -349,22 +399,28 @@ __global__ __launch_bounds__(256) void ranged_attention_tile_kernel(
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            o[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                v_lds[(nb * 16 + 4 * g4 + i) * VP + db * 16 + c16], sv[nb][i],
-                o[db], 0, 0, 0);
+          for (int i = 0; i < 4; ++i) {
+            const float a = v_lds[(nb * 16 + 4 * g4 + i) * VP + db * 16 + c16];
+#pragma unroll
+            for (int qs = 0; qs < QS; ++qs)
+              o[qs][db] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                  a, sv[qs][nb][i], o[qs][db], 0, 0, 0);
+          }
     }
     __syncthreads();
   }
 
-  if (!row_ok) return;
-  const float inv_l = 1.0f / l;
-  A* op = out + (static_cast<int64_t>(row_first + my_row) * H + h) * D;
 #pragma unroll
-  for (int db = 0; db < DB; ++db)
+  for (int qs = 0; qs < QS; ++qs) {
+    if (!row_ok[qs]) continue;
+    const float inv_l = 1.0f / l[qs];
+    A* op = out + (static_cast<int64_t>(row_first + my_row[qs]) * H + h) * D;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      Act<A>::st(op + db * 16 + 4 * g4 + i, o[db][i] * inv_l);
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        Act<A>::st(op + db * 16 + 4 * g4 + i, o[qs][db][i] * inv_l);
+  }
 }
 
 template <typename A>

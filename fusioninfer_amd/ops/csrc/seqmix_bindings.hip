@@ -256,7 +256,7 @@ void rope_unitnorm_cache(at::Tensor q_out, at::Tensor q, at::Tensor k,
 
 // Rows [0, tile_rows) belong to the row groups that the tile tables
 // cover (tile_seq/tile_row0: group and first row inside it of every
-// 64-row tile) and run the MFMA kernel when the head size has one; all
+// 128-row tile) and run the MFMA kernel when the head size has one; all
 // other rows run the row-per-wave kernel.
 void ranged_paged_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
                             at::Tensor v_cache, at::Tensor seq_bt,

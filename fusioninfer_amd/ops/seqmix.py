@@ -102,7 +102,7 @@ def rope_unitnorm_cache_(q, k, positions, inv_freq, eps: float, k_cache,
                                     num_kv_heads, head_dim)
 
 
-ATTENTION_TILE_ROWS = 64  # q rows per workgroup of the tiled kernel
+ATTENTION_TILE_ROWS = 128  # q rows per workgroup of the tiled kernel
 
 
 def build_attention_tiles(group_lens, device=None):
