@@ -151,9 +151,16 @@ __global__ __launch_bounds__(64 * kDeltaWaves) void delta_rule_wave_kernel(
       const int f = tid + NT * x;              // float4 index in the block
       if (f < BLKF4) {
         const int tt = f / TOKF4, within = f % TOKF4;
-        const int t = min(tb0 + tt, row1 - 1);  // tail: re-read the last row
-        nx[x] = *reinterpret_cast<const float4*>(vhead + t * tok_stride +
-                                                 within * 4);
+        const int t = tb0 + tt;
+        if (t < row1) {
+          nx[x] = *reinterpret_cast<const float4*>(vhead + t * tok_stride +
+                                                   within * 4);
+        } else {
+          // past the group's end: the identity token (w = 1, rest 0)
+          // leaves the state untouched, so the apply loop needs no branch
+          const float one = within < DK / 4 ? 1.f : 0.f;
+          nx[x] = float4{one, one, one, one};
+        }
       }
     }
 #pragma unroll
@@ -185,7 +192,7 @@ __global__ __launch_bounds__(64 * kDeltaWaves) void delta_rule_wave_kernel(
     const int nt = min(TB, row1 - tb0);
 #pragma unroll
     for (int tt = 0; tt < TB; ++tt) {
-      if (tt < nt) {
+      {
         const float* base = &lds[buf][tt * 5 * DK + i0];
         float4 ww[R4], au[R4], uu[R4], kk[R4], rr[R4];
 #pragma unroll
@@ -222,7 +229,7 @@ __global__ __launch_bounds__(64 * kDeltaWaves) void delta_rule_wave_kernel(
           o3 += S[4 * x + 3] * rr[x].w;
         }
         const float oc = slice_sum<SL>((o0 + o1) + (o2 + o3));
-        if (slice == 0 && col_ok)
+        if (slice == 0 && col_ok && tt < nt)
           o_raw[static_cast<int64_t>(tb0 + tt) * heads * dim + hbase + c] = oc;
       }
     }
