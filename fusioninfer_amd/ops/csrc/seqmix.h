@@ -24,6 +24,43 @@ struct Act<u16> {
   static FI_DEV void st(u16* p, float v) { *p = f32_to_bf16(v); }
 };
 
+// VW consecutive activations (VW = 1, or 4 with one 16-/8-byte access)
+template <typename A, int VW>
+FI_DEV void ldv(const A* p, float* v);
+template <typename A, int VW>
+FI_DEV void stv(A* p, const float* v);
+
+template <>
+FI_DEV void ldv<float, 1>(const float* p, float* v) { v[0] = *p; }
+template <>
+FI_DEV void ldv<u16, 1>(const u16* p, float* v) { v[0] = bf16_to_f32(*p); }
+template <>
+FI_DEV void ldv<float, 4>(const float* p, float* v) {
+  const float4 x = *reinterpret_cast<const float4*>(p);
+  v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+}
+template <>
+FI_DEV void ldv<u16, 4>(const u16* p, float* v) {
+  const bf16x4 x = *reinterpret_cast<const bf16x4*>(p);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = bf16_to_f32(x.h[i]);
+}
+template <>
+FI_DEV void stv<float, 1>(float* p, const float* v) { *p = v[0]; }
+template <>
+FI_DEV void stv<u16, 1>(u16* p, const float* v) { *p = f32_to_bf16(v[0]); }
+template <>
+FI_DEV void stv<float, 4>(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = float4{v[0], v[1], v[2], v[3]};
+}
+template <>
+FI_DEV void stv<u16, 4>(u16* p, const float* v) {
+  bf16x4 x;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) x.h[i] = f32_to_bf16(v[i]);
+  *reinterpret_cast<bf16x4*>(p) = x;
+}
+
 // Sum of two values over a 256-thread block at once (one barrier pair).
 // scratch: 8 floats. Safe to call repeatedly with the same scratch.
 FI_DEV void block_reduce_sum2_256(float& a, float& b, float* scratch) {

@@ -36,7 +36,7 @@ def _native():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("W", [96, 256, 1000])
+@pytest.mark.parametrize("W", [96, 256, 1000, 37, 2050])
 def test_row_norms(dtype, W):
     torch.manual_seed(0)
     dev = "cuda"
