@@ -157,7 +157,7 @@ def test_token_shift_and_scalar_norm(device):
 
 
 def _attention_case(device, dim, rot, chunk, T, H=2, G=1, pos0=0, seed=0,
-                    boost=None):
+                    boost=None, decode_tail=0):
     """Product attention (cache write + ranged attention) on one sequence
     fed as two portions, against the oracle's whole-sequence attention.
     boost=(i, j): query i and key j get one large shared direction so the
@@ -193,7 +193,11 @@ def _attention_case(device, dim, rot, chunk, T, H=2, G=1, pos0=0, seed=0,
     k = (h @ Wk.T).float().to(device)
     outs = []
     cut = T // 2 + 1
-    for a, b in ((0, cut), (cut, T)):
+    spans = [(0, cut), (cut, T - decode_tail)]
+    spans += [(t, t + 1) for t in range(T - decode_tail, T)]  # one by one
+    for a, b in spans:
+        if b <= a:
+            continue
         pos = list(range(a, b))
         slots = [blocks[p // bs] * bs + p % bs for p in pos]
         qn = seqmix.rope_unitnorm_cache_(q[a:b], k[a:b], mk(pos), inv, 1e-3,
@@ -201,7 +205,8 @@ def _attention_case(device, dim, rot, chunk, T, H=2, G=1, pos0=0, seed=0,
         outs.append(seqmix.ranged_paged_attention(
             qn.view(b - a, H, dim), kc, vc, bt, mk([0] * (b - a)), mk(pos),
             0.4, chunk=chunk, seq_cu=mk([0, b - a]),
-            tiles=seqmix.build_attention_tiles([b - a], device=device)))
+            tiles=(seqmix.build_attention_tiles([b - a], device=device)
+                   if b - a > 1 else None)))
     got = torch.cat(outs).reshape(T, H * dim).cpu().double()
     return got, want
 
@@ -225,11 +230,28 @@ def test_chunk_edge_one_key_in_or_out(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+def test_chunk_edge_while_decoding(device):
+    """Same edges with the last rows fed one token at a time: the decode
+    row that opens a chunk sees only itself, the next one sees exactly
+    two keys, and a row deep in a chunk still finds the chunk's first
+    key but not the key before it."""
+    for boost in [(40, 39), (41, 40), (41, 39), (59, 40), (59, 39)]:
+        got, want = _attention_case(device, 16, 16, 20, T=60, boost=boost,
+                                    seed=3 + boost[0] + boost[1],
+                                    decode_tail=22)
+        assert (got - want).abs().max() < 2e-5, boost
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_far_key_among_hundreds(device):
     """One early key shares the last row's direction: with a chunk as
     long as the sequence it must dominate, across many pages."""
     got, want = _attention_case(device, 16, 8, 1000, T=300, boost=(299, 3),
                                 seed=5)
+    assert (got - want).abs().max() < 2e-5
+    # and for a decoded row (last 5 rows one by one)
+    got, want = _attention_case(device, 16, 8, 1000, T=300, boost=(299, 3),
+                                seed=6, decode_tail=5)
     assert (got - want).abs().max() < 2e-5
 
 
@@ -551,3 +573,27 @@ def test_gpu_engine_matches_cpu_engine_at_larger_sizes(dtype):
         e = rel_err(torch.stack([got[rid][p] for p in ps]),
                     torch.stack([want[rid][p] for p in ps]))
         assert e < lim, (rid, e)
+
+
+def test_forced_steps_serve_the_transformer_family_too():
+    """forced_step is the engine's own batch path: on the built-in
+    transformer its logits reproduce what greedy generation picks."""
+    mc = registry.get_model_config("tiny-qwen3")
+    cfg = EngineConfig(model=mc, cache=CacheConfig(num_gpu_blocks=64),
+                       scheduler=SchedulerConfig(max_num_seqs=4,
+                                                 max_model_len=512),
+                       enforce_eager=True, seed=3)
+    eng = LLMEngine(cfg, device="cpu")
+    prompt = tokens(19, 77, vocab=1000)
+    out = eng.generate([prompt], SamplingParams(max_tokens=5))[0]
+    toks = prompt + out.output_token_ids
+    # prompt in two portions, then the generated tokens one at a time
+    lg = [eng.forced_step([("x", toks[:11], [])]),
+          eng.forced_step([("x", toks[11:19], [7])])]
+    picked = [int(lg[1][0].argmax())]
+    for i in range(19, 23):
+        picked.append(int(eng.forced_step([("x", [toks[i]], [0])])[0]
+                          .argmax()))
+    eng.forced_step([], ["x"])
+    assert picked == out.output_token_ids
+    assert eng.block_manager.num_free() == 64
