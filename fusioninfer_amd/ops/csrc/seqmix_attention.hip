@@ -275,24 +275,48 @@ __global__ __launch_bounds__(256) void ranged_attention_tile_kernel(
   for (int j0 = kv_lo; j0 <= kv_hi; j0 += BN) {
     // ---- stage K and V tiles (zero-filled past the range) ----
     constexpr int VPR = D / VEC;               // vectors per key row
-    for (int vid = tid; vid < BN * VPR; vid += 256) {
-      const int key_l = vid / VPR, dv = vid % VPR;
-      const int key = j0 + key_l;
-      typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
-      u32x4 kv4 = {0u, 0u, 0u, 0u}, vv4 = {0u, 0u, 0u, 0u};
-      if (key <= kv_hi) {
-        const int64_t off =
-            ((static_cast<int64_t>(bt[key / block_size]) * G + g) * block_size +
-             key % block_size) * D + dv * VEC;
-        kv4 = *reinterpret_cast<const u32x4*>(k_cache + off);
-        vv4 = *reinterpret_cast<const u32x4*>(v_cache + off);
-      }
-      *reinterpret_cast<u32x4*>(k_lds + key_l * KP + dv * VEC) = kv4;
-      if constexpr (BF) {
-        const u16* ve = reinterpret_cast<const u16*>(&vv4);
+    typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+    if constexpr (BF) {
+      // two adjacent keys per thread: the transposed V tile is written
+      // with 4-byte stores (one (key, key+1) pair per d)
+      for (int pid = tid; pid < (BN / 2) * VPR; pid += 256) {
+        const int kp = pid / VPR, dv = pid % VPR;
+        u32x4 k4[2], v4[2];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v_lds[(dv * 8 + e) * VP + key_l] = ve[e];
-      } else {
+        for (int e2 = 0; e2 < 2; ++e2) {
+          const int key = j0 + 2 * kp + e2;
+          k4[e2] = u32x4{0u, 0u, 0u, 0u};
+          v4[e2] = u32x4{0u, 0u, 0u, 0u};
+          if (key <= kv_hi) {
+            const int64_t off =
+                ((static_cast<int64_t>(bt[key / block_size]) * G + g) *
+                     block_size + key % block_size) * D + dv * VEC;
+            k4[e2] = *reinterpret_cast<const u32x4*>(k_cache + off);
+            v4[e2] = *reinterpret_cast<const u32x4*>(v_cache + off);
+          }
+          *reinterpret_cast<u32x4*>(k_lds + (2 * kp + e2) * KP + dv * VEC) =
+              k4[e2];
+        }
+        const u16* va = reinterpret_cast<const u16*>(&v4[0]);
+        const u16* vb = reinterpret_cast<const u16*>(&v4[1]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          *reinterpret_cast<u32*>(v_lds + (dv * 8 + e) * VP + 2 * kp) =
+              static_cast<u32>(va[e]) | (static_cast<u32>(vb[e]) << 16);
+      }
+    } else {
+      for (int vid = tid; vid < BN * VPR; vid += 256) {
+        const int key_l = vid / VPR, dv = vid % VPR;
+        const int key = j0 + key_l;
+        u32x4 kv4 = {0u, 0u, 0u, 0u}, vv4 = {0u, 0u, 0u, 0u};
+        if (key <= kv_hi) {
+          const int64_t off =
+              ((static_cast<int64_t>(bt[key / block_size]) * G + g) *
+                   block_size + key % block_size) * D + dv * VEC;
+          kv4 = *reinterpret_cast<const u32x4*>(k_cache + off);
+          vv4 = *reinterpret_cast<const u32x4*>(v_cache + off);
+        }
+        *reinterpret_cast<u32x4*>(k_lds + key_l * KP + dv * VEC) = kv4;
         *reinterpret_cast<u32x4*>(v_lds + key_l * VP + dv * VEC) = vv4;
       }
     }
