@@ -80,7 +80,7 @@ def safetensors_shapes(path: str) -> Dict[str, Tuple[int, ...]]:
 
 
 def parse_config(raw: dict, shapes: Optional[Dict[str, tuple]] = None,
-                 default_decay_rank: int = 16) -> PinuvikConfig:
+                 default_decay_rank: int = 32) -> PinuvikConfig:
     """config.json -> PinuvikConfig. Sizes the config does not carry (the
     inner size of the decay branch) come from the checkpoint's tensor
     shapes, or from an optional ``decay_rank`` key for random-init use."""

@@ -597,3 +597,19 @@ def test_forced_steps_serve_the_transformer_family_too():
     eng.forced_step([], ["x"])
     assert picked == out.output_token_ids
     assert eng.block_manager.num_free() == 64
+
+
+@pytest.mark.gpu
+def test_generation_with_graph_replay_and_pipelined_decode():
+    """engine.generate on the GPU with captured decode graphs: admission,
+    chunked prefill, graph replays fed by on-device sampled ids, slot
+    recycling (more prompts than slots) - token-exact with the oracle."""
+    raw = small_config()
+    eng, W = make_engine(raw, "cuda", eager=False, max_seqs=2, budget=16,
+                         seed=9)
+    assert eng.runner._graphs
+    prompts = [tokens(21, 51), tokens(5, 52), tokens(33, 53), tokens(2, 54)]
+    outs = eng.generate(prompts, SamplingParams(max_tokens=10))
+    for p, o in zip(prompts, outs):
+        assert o.output_token_ids == oracle.greedy(raw, W, p, 10)
+    assert eng.state_manager.num_free() == 2
