@@ -14,6 +14,24 @@ model designs assemble them freely:
   merged input projection; the halves are width-normalized and averaged by
   the caller's fused residual kernel.
 * ``GatedMLP``           act(gate) * up -> down with a chosen activation.
+* ``DecayLinearAttention``  linear attention with one scalar decay per
+  head (silu feature maps), fp32 state in the state slots, whole-row
+  unit-RMS output with gain and sigmoid gate.
+* ``TalkingWindowAttention``  grouped-query softmax attention without
+  rotation: projection biases, a log-distance score penalty per head,
+  scores mixed across heads before the softmax, sliding window; separate
+  key and value sizes in the paged cache.
+* ``GatedDeltaMixer``    gated delta rule (scalar decay and write strength
+  per head and token) behind a short causal convolution whose tail is
+  part of the slot state; per-head unit-RMS output with a shared gain and
+  a silu gate.
+* ``RoutedExperts``      mixture of gated feed-forward experts with a
+  sigmoid or softmax router, top-k choice, optional renormalisation and a
+  constant factor on the weights.
+* ``GatedResidualLayer`` layer-normed residual layer whose sublayer
+  results are multiplied by sigmoid(W h + b) before they are added; one
+  mixer or several scaled mixers side by side behind ONE merged input
+  projection (which also carries the gate's W).
 
 Activations run in the model dtype (bf16 or fp32); statistics, rotary
 angles, scores, decays, gates of the recurrence and the state are fp32
@@ -24,10 +42,11 @@ from __future__ import annotations
 
 import dataclasses
 import math
-from typing import List, Optional
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from fusioninfer_amd.distributed.layers import (
     MergedColumnParallelLinear,
@@ -233,3 +252,363 @@ class MixerLayer(nn.Module):
             seqmix.residual_add_scalar_norm_(
                 resid, self.mlp(h2), self.norm2b, self.eps)
         return resid
+
+
+# ------------------------------------------------------------------------
+# Layer-norm / gated-residual family of blocks
+
+
+@dataclasses.dataclass
+class DecayLinearAttentionConfig:
+    heads: int
+    dim: int                 # per-head query/key size
+    vdim: int                # per-head value size
+    decay: Tuple[float, ...]  # one factor per head
+
+    def __post_init__(self):
+        if len(self.decay) != self.heads:
+            raise ValueError("one decay per head is needed "
+                             f"(got {len(self.decay)} for {self.heads})")
+
+
+@dataclasses.dataclass
+class TalkingWindowAttentionConfig:
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int = 0          # >0: keys only from the last `window` positions
+
+    def __post_init__(self):
+        if self.heads % self.kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+
+
+@dataclasses.dataclass
+class GatedDeltaConfig:
+    heads: int               # value heads (= state heads)
+    kv_heads: int            # query/key heads
+    dim: int
+    vdim: int
+    conv: int                # taps of the causal convolution (1 = none)
+
+    def __post_init__(self):
+        if self.heads % self.kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        if self.conv < 1:
+            raise ValueError("conv taps must be >= 1")
+
+
+def _f32_rand(shape, lo: float, hi: float) -> nn.Parameter:
+    return nn.Parameter(
+        torch.rand(shape, dtype=torch.float32) * (hi - lo) + lo,
+        requires_grad=False)
+
+
+class DecayLinearAttention(nn.Module):
+    """Linear-attention mixer: consumes its slice of the merged projection
+    (q, k, v, output gate)."""
+
+    has_bias = False
+
+    def __init__(self, cfg: DecayLinearAttentionConfig, width: int,
+                 eps: float, dtype):
+        super().__init__()
+        self.cfg = cfg
+        self.eps = eps
+        self.dtype = dtype
+        n, nv = cfg.heads * cfg.dim, cfg.heads * cfg.vdim
+        self.in_sizes = [n, n, nv, nv]
+        self.in_names = ["q", "k", "v", "g"]
+        self.register_buffer(
+            "decay", torch.tensor(cfg.decay, dtype=torch.float32),
+            persistent=False)
+        self.norm_w = _f32_param((nv,), 1.0)
+        self.o_proj = RowParallelLinear(nv, width, dtype=dtype)
+
+    def state_tensors(self, num_blocks, block_size, num_slots, device):
+        c = self.cfg
+        return {"lin": torch.zeros((num_slots, c.heads, c.dim, c.vdim),
+                                   dtype=torch.float32, device=device)}
+
+    def block_bytes(self, block_size: int) -> int:
+        return 0
+
+    def forward(self, parts, meta, cache) -> torch.Tensor:
+        q, k, v, g = parts
+        c = self.cfg
+        o_raw = seqmix.decay_linear_attention(
+            q, k, v, self.decay, cache["lin"], meta.seq_cu, meta.seq_slots,
+            meta.positions, c.heads, c.dim, c.vdim)
+        o = seqmix.group_rms_gate(o_raw, g, self.norm_w, 1, self.eps,
+                                  "sigmoid", self.dtype)
+        return self.o_proj(o)
+
+
+class TalkingWindowAttention(nn.Module):
+    """Windowed softmax attention with head mixing; q/k/v biases ride the
+    merged projection's bias."""
+
+    has_bias = True
+
+    def __init__(self, cfg: TalkingWindowAttentionConfig, width: int,
+                 eps: float, dtype):
+        super().__init__()
+        self.cfg = cfg
+        self.dtype = dtype
+        self.in_sizes = [cfg.heads * cfg.dim, cfg.kv_heads * cfg.dim,
+                         cfg.kv_heads * cfg.vdim]
+        self.in_names = ["q", "k", "v"]
+        self.r1 = _f32_param((cfg.heads,), 0.0)
+        self.r2 = _f32_param((cfg.heads,), 0.0)
+        self.talk = nn.Parameter(torch.eye(cfg.heads, dtype=torch.float32),
+                                 requires_grad=False)
+        self.o_proj = RowParallelLinear(cfg.heads * cfg.vdim, width,
+                                        dtype=dtype)
+        self.o_bias = nn.Parameter(torch.zeros(width, dtype=dtype),
+                                   requires_grad=False)
+
+    def state_tensors(self, num_blocks, block_size, num_slots, device):
+        c = self.cfg
+        return {
+            "k": torch.zeros((num_blocks, c.kv_heads, block_size, c.dim),
+                             dtype=self.dtype, device=device),
+            "v": torch.zeros((num_blocks, c.kv_heads, block_size, c.vdim),
+                             dtype=self.dtype, device=device),
+        }
+
+    def block_bytes(self, block_size: int) -> int:
+        c = self.cfg
+        esize = torch.empty((), dtype=self.dtype).element_size()
+        return c.kv_heads * block_size * (c.dim + c.vdim) * esize
+
+    def forward(self, parts, meta, cache) -> torch.Tensor:
+        q, k, v = parts
+        c = self.cfg
+        seqmix.paged_cache_write_(k, v, cache["k"], cache["v"],
+                                  meta.slot_mapping)
+        o = seqmix.talking_window_attention(
+            q, cache["k"], cache["v"], meta.seq_bt, meta.row_seq,
+            meta.positions, c.scale, c.window, self.r1, self.r2, self.talk,
+            c.heads, seq_cu=meta.seq_cu, tiles=meta.seq_tiles)
+        return F.linear(o.view(o.shape[0], c.heads * c.vdim),
+                        self.o_proj.weight, self.o_bias)
+
+
+class GatedDeltaMixer(nn.Module):
+    """Gated-delta-rule mixer: q, k, v (convolved), write strength, decay
+    input and output gate come from the merged projection."""
+
+    has_bias = False
+
+    def __init__(self, cfg: GatedDeltaConfig, width: int, eps: float, dtype):
+        super().__init__()
+        self.cfg = cfg
+        self.eps = eps
+        self.dtype = dtype
+        nq, nv = cfg.kv_heads * cfg.dim, cfg.heads * cfg.vdim
+        self.channels = 2 * nq + nv
+        # q | k | v stay adjacent: the convolution reads them as one block
+        self.in_sizes = [nq, nq, nv, cfg.heads, cfg.heads, nv]
+        self.in_names = ["q", "k", "v", "b", "a", "g"]
+        conv = torch.zeros(self.channels, cfg.conv, dtype=torch.float32)
+        conv[:, -1] = 1.0
+        self.conv_w = nn.Parameter(conv, requires_grad=False)
+        self.a_log = _f32_param((cfg.heads,), 0.0)
+        self.dt_bias = _f32_param((cfg.heads,), 0.0)
+        self.norm_w = _f32_param((cfg.vdim,), 1.0)
+        self.o_proj = RowParallelLinear(nv, width, dtype=dtype)
+
+    def state_tensors(self, num_blocks, block_size, num_slots, device):
+        c = self.cfg
+        return {
+            "conv": torch.zeros((num_slots, max(c.conv - 1, 1), self.channels),
+                                dtype=torch.float32, device=device),
+            "delta": torch.zeros((num_slots, c.heads, c.dim, c.vdim),
+                                 dtype=torch.float32, device=device),
+        }
+
+    def block_bytes(self, block_size: int) -> int:
+        return 0
+
+    def forward(self, parts, meta, cache) -> torch.Tensor:
+        q, k, v, b, a, g = parts
+        c = self.cfg
+        # q|k|v as one strided view of the projection output
+        x = torch.as_strided(
+            q, (q.shape[0], self.channels), (q.stride(0), 1),
+            q.storage_offset())
+        o_raw = seqmix.gated_delta_rule(
+            x, self.conv_w, a, b, self.a_log, self.dt_bias, cache["conv"],
+            cache["delta"], meta.seq_cu, meta.seq_slots, meta.positions,
+            c.heads, c.kv_heads, c.dim, c.vdim, row_seq=meta.row_seq)
+        o = seqmix.group_rms_gate(o_raw, g, self.norm_w, c.heads, self.eps,
+                                  "silu", self.dtype)
+        return self.o_proj(o)
+
+
+class RoutedExperts(nn.Module):
+    """Mixture of gated feed-forward experts: down(silu(gate x) * up x).
+
+    Router logits are an fp32 product; scores are sigmoid(z) or
+    softmax(z); the ``top`` largest are chosen, optionally divided by their
+    sum (+1e-20), and multiplied by ``scale``. On the GPU the experts run
+    as two grouped GEMMs over block-aligned expert segments: the MFMA
+    kernel on packed bf16 weights where the sizes fit its tiles, the
+    plain grouped kernel otherwise (fp32, odd sizes)."""
+
+    def __init__(self, width: int, ff: int, experts: int, top: int, dtype,
+                 score: str = "sigmoid", renorm: bool = True,
+                 scale: float = 1.0):
+        super().__init__()
+        if score not in ("sigmoid", "softmax"):
+            raise ValueError(f"unknown router score {score!r}")
+        if not 1 <= top <= experts:
+            raise ValueError("top must be in 1..experts")
+        self.width, self.ff, self.experts, self.top = width, ff, experts, top
+        self.score, self.renorm, self.scale = score, renorm, float(scale)
+        self.dtype = dtype
+        self.router = nn.Parameter(
+            torch.empty(experts, width, dtype=torch.float32).normal_(0, 0.02),
+            requires_grad=False)
+        self.gate_up = nn.Parameter(
+            torch.empty(experts, 2 * ff, width, dtype=dtype).normal_(0, 0.02),
+            requires_grad=False)
+        self.down = nn.Parameter(
+            torch.empty(experts, width, ff, dtype=dtype).normal_(0, 0.02),
+            requires_grad=False)
+        self._packed = None
+
+    # the MFMA grouped GEMM wants bf16, K % 32 == 0 and whole column tiles
+    def _mfma_fits(self) -> bool:
+        return (self.dtype == torch.bfloat16 and self.width % 128 == 0
+                and self.ff % 64 == 0 and self.experts <= 128)
+
+    def invalidate_packed(self):
+        self._packed = None
+
+    def _packed_weights(self):
+        if self._packed is None:
+            from fusioninfer_amd import ops
+
+            self._packed = (
+                ops.pack_moe_weights(
+                    self.gate_up.data.transpose(1, 2).contiguous()),
+                ops.pack_moe_weights(
+                    self.down.data.transpose(1, 2).contiguous()))
+        return self._packed
+
+    def route(self, x):
+        from fusioninfer_amd import ops
+
+        logits = F.linear(x.float(), self.router)
+        return ops.moe_route(logits, self.top, self.score, self.renorm,
+                             self.scale)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        from fusioninfer_amd import ops
+
+        T = x.shape[0]
+        topv, topi = self.route(x)
+        if not x.is_cuda:
+            out = torch.zeros(T, self.width, dtype=torch.float32)
+            for e in range(self.experts):
+                rows, kk = (topi == e).nonzero(as_tuple=True)
+                if rows.numel() == 0:
+                    continue
+                gu = F.linear(x[rows], self.gate_up[e]).float()
+                act = (F.silu(gu[:, : self.ff]) * gu[:, self.ff:]).to(x.dtype)
+                y = F.linear(act, self.down[e]).float()
+                out.index_add_(0, rows, y * topv[rows, kk].unsqueeze(1))
+            return out.to(x.dtype)
+        E = self.experts
+        fast = self._mfma_fits()
+        block_m = 16
+        if fast and T * self.top >= 64 * E:
+            block_m = 128
+        sorted_ids, expert_ids, n_valid, pos, PM = ops.moe_align(
+            topi, 0, E, block_m)
+        act = torch.empty(PM, self.ff, dtype=x.dtype, device=x.device)
+        y = torch.empty(PM, self.width, dtype=x.dtype, device=x.device)
+        if fast:
+            gu_p, dn_p = self._packed_weights()
+            ops.moe_gemm(act, x, gu_p, sorted_ids, expert_ids, n_valid,
+                         block_m, gate_up=True)
+            ops.moe_gemm(y, act, dn_p, sorted_ids, expert_ids, n_valid,
+                         block_m, gate_up=False)
+        else:
+            ops.moe_gemm_plain(act, x, self.gate_up, sorted_ids, expert_ids,
+                               n_valid, block_m, gate_up=True)
+            ops.moe_gemm_plain(y, act, self.down, sorted_ids, expert_ids,
+                               n_valid, block_m, gate_up=False)
+        out = torch.empty(T, self.width, dtype=x.dtype, device=x.device)
+        ops.moe_combine(out, y, pos, topv.reshape(-1).contiguous())
+        return out
+
+
+class GatedResidualLayer(nn.Module):
+    """x <- x + gate1 * sum_m scale_m mixer_m(h),  h = layer_norm(x) w1
+    x <- x + gate2 * ff(h2),                       h2 = layer_norm(x) w2
+    with gate = sigmoid(W h + b) per coordinate and the residual stream x
+    kept in fp32. All input branches of all mixers and the first gate's W
+    are one merged projection of h. ``forward`` receives h (this layer's
+    normed input) and returns the NEXT layer's normed input, so every
+    residual update is fused with the norm that follows it."""
+
+    def __init__(self, mixers: Sequence[Tuple[str, nn.Module, float]],
+                 mlp: Optional[nn.Module], width: int, eps: float, dtype):
+        super().__init__()
+        if not 1 <= len(mixers) <= 2:
+            raise ValueError("one or two mixers per layer")
+        self.names = [m[0] for m in mixers]
+        self.mixers = nn.ModuleList([m[1] for m in mixers])
+        self.scales = [float(m[2]) for m in mixers]
+        self.mlp = mlp
+        self.eps = eps
+        self.dtype = dtype
+        self.width = width
+        self.branches: List[Tuple[str, str]] = []
+        self.sizes: List[int] = []
+        for name, mod in zip(self.names, self.mixers):
+            for br, size in zip(mod.in_names, mod.in_sizes):
+                self.branches.append((name, br))
+                self.sizes.append(size)
+        self.branches.append(("", "rg1"))
+        self.sizes.append(width)
+        self.in_proj = MergedColumnParallelLinear(
+            width, self.sizes, dtype=dtype,
+            bias=any(m.has_bias for m in self.mixers))
+        self.norm1 = _f32_param((width,), 1.0)
+        self.rg1_bias = _f32_param((width,), 0.0)
+        if mlp is not None:
+            self.norm2 = _f32_param((width,), 1.0)
+            self.rg2 = ReplicatedLinear(width, width, dtype=dtype)
+            self.rg2_bias = _f32_param((width,), 0.0)
+
+    def in_proj_rows(self, mixer: str, branch: str):
+        off = 0
+        for key, size in zip(self.branches, self.sizes):
+            if key == (mixer, branch):
+                return off, size
+            off += size
+        raise KeyError((mixer, branch))
+
+    def forward(self, resid, h, meta, cache, next_norm_w):
+        parts = self.in_proj(h).split(self.sizes, dim=-1)
+        ys, at = [], 0
+        for mod in self.mixers:
+            n = len(mod.in_sizes)
+            ys.append(mod(parts[at: at + n], meta, cache))
+            at += n
+        w_after = self.norm2 if self.mlp is not None else next_norm_w
+        h2 = seqmix.gated_residual_layer_norm_(
+            resid, ys[0], self.scales[0],
+            ys[1] if len(ys) > 1 else None,
+            self.scales[1] if len(ys) > 1 else 0.0,
+            parts[-1], self.rg1_bias, w_after, self.eps, self.dtype)
+        if self.mlp is None:
+            return h2
+        return seqmix.gated_residual_layer_norm_(
+            resid, self.mlp(h2), 1.0, None, 0.0, self.rg2(h2), self.rg2_bias,
+            next_norm_w, self.eps, self.dtype)

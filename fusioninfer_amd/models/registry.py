@@ -211,10 +211,21 @@ register(
 _ARCHITECTURES = {}
 
 
-def register_architecture(name: str, config_from_dict, model_factory) -> None:
+def register_architecture(name: str, config_from_dict, model_factory,
+                          extensions=("seqmix",)) -> None:
     """config_from_dict(raw: dict, model_path) -> ModelConfig;
-    model_factory(cfg: ModelConfig) -> nn.Module."""
-    _ARCHITECTURES[name.lower()] = (config_from_dict, model_factory)
+    model_factory(cfg: ModelConfig) -> nn.Module; ``extensions`` names the
+    HIP extensions (ops/build.py) the family's GPU path loads."""
+    _ARCHITECTURES[name.lower()] = (config_from_dict, model_factory,
+                                    tuple(extensions))
+
+
+def required_extensions(cfg: ModelConfig):
+    """HIP extensions a model of this config runs on the GPU, so that a
+    fresh checkout compiles only those."""
+    if cfg.architecture == "transformer":
+        return ("core", "moe") if cfg.is_moe else ("core",)
+    return _ARCHITECTURES[cfg.architecture.lower()][2]
 
 
 def _register_builtin_architectures() -> None:
@@ -229,6 +240,19 @@ def _register_builtin_architectures() -> None:
         return PinuvikLM(cfg)
 
     register_architecture("Pinuvik", pinuvik_config, pinuvik_model)
+
+    def sefalorn_config(raw, model_path):
+        from fusioninfer_amd.models import sefalorn
+
+        return sefalorn.model_config_from_dict(raw, model_path)
+
+    def sefalorn_model(cfg):
+        from fusioninfer_amd.models.sefalorn import SefalornLM
+
+        return SefalornLM(cfg)
+
+    register_architecture("Sefalorn", sefalorn_config, sefalorn_model,
+                          extensions=("seqmix", "moe"))
 
 
 _register_builtin_architectures()

@@ -355,6 +355,37 @@ def pack_moe_weights(w: torch.Tensor) -> torch.Tensor:
     )
 
 
+_C_MOE = None
+_C_MOE_ERR: Optional[BaseException] = None
+
+
+def _moe_native():
+    """The expert-routing kernels live in their own extension
+    (``_C_moe.so``) so that any model family with routed experts compiles
+    only them, not the transformer kernels."""
+    global _C_MOE, _C_MOE_ERR
+    if _C_MOE is None:
+        try:
+            import importlib
+
+            _C_MOE = importlib.import_module("fusioninfer_amd.ops._C_moe")
+        except Exception as e:  # noqa: BLE001
+            _C_MOE_ERR = e
+            raise RuntimeError(
+                "fusioninfer_amd expert-routing extension (_C_moe.so) is "
+                "not available but a GPU tensor was passed; build it with "
+                "`python -m fusioninfer_amd.ops.build moe`."
+            ) from e
+    return _C_MOE
+
+
+def has_moe_native() -> bool:
+    try:
+        return _moe_native() is not None
+    except RuntimeError:
+        return False
+
+
 def moe_gemm(out, a, b_packed, sorted_ids, expert_ids, n_valid,
              block_m: int, gate_up: bool):
     """Grouped GEMM over block-aligned expert segments.
@@ -365,12 +396,22 @@ def moe_gemm(out, a, b_packed, sorted_ids, expert_ids, n_valid,
     the real m-tile count (static grid, dynamic work — hipGraph-safe).
     gate_up=True fuses the SwiGLU epilogue: out = silu(gate) * up."""
     if out.is_cuda:
-        _require_native()
-        _C.moe_gemm(out, a, b_packed, sorted_ids, expert_ids, n_valid,
-                    block_m, gate_up)
+        _moe_native().moe_gemm(out, a, b_packed, sorted_ids, expert_ids,
+                               n_valid, block_m, gate_up)
         return out
     return ref.moe_gemm(out, a, b_packed, sorted_ids, expert_ids, n_valid,
                         block_m, gate_up)
+
+
+def moe_gemm_plain(out, a, w, sorted_ids, expert_ids, n_valid, block_m: int,
+                   gate_up: bool):
+    """Grouped GEMM of the same block-aligned layout for ANY sizes and for
+    fp32 or bf16 operands (fp32 accumulation): w is the experts' natural
+    [E, out, in] weight ([E, 2N, K] with gate rows first when gate_up,
+    which also applies out = silu(gate) * up). GPU only."""
+    _moe_native().moe_gemm_plain(out, a, w, sorted_ids, expert_ids, n_valid,
+                                 block_m, gate_up)
+    return out
 
 
 def moe_gemm_fp8(out, a, a_scales, b_packed, b_scales, sorted_ids,
@@ -380,9 +421,9 @@ def moe_gemm_fp8(out, a, a_scales, b_packed, b_scales, sorted_ids,
     SwiGLU. Same block-aligned layout as moe_gemm; b_packed from
     pack_moe_weights over the [E, K, N] e4m3 weights."""
     if out.is_cuda:
-        _require_native()
-        _C.moe_gemm_fp8(out, a, a_scales, b_packed, b_scales, sorted_ids,
-                        expert_ids, n_valid, block_m, gate_up)
+        _moe_native().moe_gemm_fp8(out, a, a_scales, b_packed, b_scales,
+                                   sorted_ids, expert_ids, n_valid, block_m,
+                                   gate_up)
         return out
     return ref.moe_gemm_fp8(out, a, a_scales, b_packed, b_scales,
                             sorted_ids, expert_ids, n_valid, block_m,
@@ -397,7 +438,7 @@ def moe_align(topi: torch.Tensor, e_start: int, e_end: int, block_m: int):
     bit-identical either way (each row's K-loop and the pos-gathered
     combine don't depend on the slot). Returns
     (sorted_ids [PM], expert_ids [PM/bm], n_valid [1], pos [T*k], PM)."""
-    _require_native()
+    C = _moe_native()
     T, k = topi.shape
     n = T * k
     E_local = e_end - e_start
@@ -407,8 +448,8 @@ def moe_align(topi: torch.Tensor, e_start: int, e_end: int, block_m: int):
     expert_ids = torch.empty(PM // block_m, dtype=torch.int32, device=dev)
     n_valid = torch.empty(1, dtype=torch.int32, device=dev)
     pos = torch.empty(n, dtype=torch.int32, device=dev)
-    _C.moe_align(topi.reshape(-1).int().contiguous(), sorted_ids,
-                 expert_ids, n_valid, pos, k, e_start, e_end, block_m)
+    C.moe_align(topi.reshape(-1).int().contiguous(), sorted_ids,
+                expert_ids, n_valid, pos, k, e_start, e_end, block_m)
     return sorted_ids, expert_ids, n_valid, pos, PM
 
 
@@ -417,20 +458,38 @@ def moe_router_topk(logits: torch.Tensor, k: int, renorm: bool):
     renormalization in one wave-per-token kernel. logits [T, E] fp32;
     returns (topv [T,k] fp32 weights, topi [T,k] int32 expert ids,
     descending; ties pick the smaller index)."""
-    _require_native()
+    C = _moe_native()
     T, E = logits.shape
     topv = torch.empty(T, k, dtype=torch.float32, device=logits.device)
     topi = torch.empty(T, k, dtype=torch.int32, device=logits.device)
-    _C.moe_router_topk(logits.contiguous(), topv, topi, k, renorm)
+    C.moe_router_topk(logits.contiguous(), topv, topi, k, renorm)
     return topv, topi
+
+
+def moe_route(logits: torch.Tensor, k: int, score: str = "softmax",
+              renorm: bool = True, scale: float = 1.0):
+    """Router tail for any expert count: scores = softmax(logits) or
+    sigmoid(logits) in fp32, the k largest chosen (ties: smaller index),
+    weights = chosen scores, divided by their sum + 1e-20 when ``renorm``,
+    times ``scale``. Returns (weights [T,k] fp32, ids [T,k] int32)."""
+    if score not in ("softmax", "sigmoid"):
+        raise ValueError(f"unknown router score {score!r}")
+    if logits.is_cuda:
+        T, E = logits.shape
+        topv = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+        topi = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+        _moe_native().moe_route(logits.contiguous(), topv, topi, k,
+                                score == "sigmoid", renorm, float(scale))
+        return topv, topi
+    return ref.moe_route(logits, k, score, renorm, scale)
 
 
 def moe_combine(out, y, pos, w):
     """out[t] = sum_k w[t,k] * y[pos[t,k]] (pos < 0 skipped). Deterministic
-    (no atomics) so token-exact tests stay reproducible."""
+    (no atomics) so token-exact tests stay reproducible. bf16 or fp32
+    rows of any width."""
     if out.is_cuda:
-        _require_native()
-        _C.moe_combine(out, y, pos, w)
+        _moe_native().moe_combine(out, y, pos, w)
         return out
     return ref.moe_combine(out, y, pos, w)
 

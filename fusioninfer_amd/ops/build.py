@@ -5,10 +5,11 @@ resulting ``_C.so`` lives next to this file so the gpurun snapshot carries it.
 
 Two extensions, so that a model family compiles only what it runs:
 
-  core    -> _C.so         transformer / MoE kernels
+  core    -> _C.so         transformer kernels
   seqmix  -> _C_seqmix.so  sequence-mixer kernels (ops/seqmix.py)
+  moe     -> _C_moe.so     expert-routing kernels (ops.moe_*)
 
-Usage:  python -m fusioninfer_amd.ops.build [core|seqmix|all] [--force]
+Usage:  python -m fusioninfer_amd.ops.build [core|seqmix|moe|all] [--force]
 """
 
 from __future__ import annotations
@@ -31,7 +32,12 @@ SOURCES = [
     "cache.hip",
     "paged_attention.hip",
     "prefill_attention.hip",
+]
+
+MOE_SOURCES = [
+    "moe_bindings.hip",
     "moe_gemm.hip",
+    "moe_plain.hip",
 ]
 
 
@@ -40,11 +46,14 @@ SEQMIX_SOURCES = [
     "seqmix_norm.hip",
     "seqmix_attention.hip",
     "seqmix_delta.hip",
+    "seqmix_stream.hip",
+    "seqmix_window.hip",
 ]
 
 EXTENSIONS = {
     "core": ("_C", SOURCES, ["common.h"]),
     "seqmix": ("_C_seqmix", SEQMIX_SOURCES, ["common.h", "seqmix.h"]),
+    "moe": ("_C_moe", MOE_SOURCES, ["common.h", "seqmix.h"]),
 }
 
 

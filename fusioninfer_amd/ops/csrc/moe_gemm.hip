@@ -468,33 +468,6 @@ __global__ __launch_bounds__(256) void moe_gemm_fp8_kernel(
   }
 }
 
-// out[t, :] = sum_k w[t,k] * y[pos[t,k], :]   (pos < 0 -> non-local expert
-// or padding: skipped). Deterministic — no atomics, so token-exact TP/PD
-// tests stay reproducible.
-__global__ void moe_combine_kernel(u16* __restrict__ out,
-                                   const u16* __restrict__ y,
-                                   const int* __restrict__ pos,
-                                   const float* __restrict__ w,
-                                   const int topk, const int H) {
-  const int t = blockIdx.y;
-  const int c0 = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
-  if (c0 + 8 > H) return;
-  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int k = 0; k < topk; ++k) {
-    const int p = pos[t * topk + k];
-    if (p < 0) continue;
-    const float wk = w[t * topk + k];
-    const bf16x8 v = *reinterpret_cast<const bf16x8*>(
-        y + static_cast<int64_t>(p) * H + c0);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] += wk * bf16_to_f32(v.h[i]);
-  }
-  bf16x8 o;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) o.h[i] = f32_to_bf16(acc[i]);
-  *reinterpret_cast<bf16x8*>(out + static_cast<int64_t>(t) * H + c0) = o;
-}
-
 }  // namespace
 
 // block_m 16: decode regime (few rows per expert; WM=1,WN=4,MITER=1 —
@@ -591,20 +564,11 @@ void launch_moe_gemm_fp8(u16* out, const unsigned char* a,
   }
 }
 
-void launch_moe_combine(u16* out, const u16* y, const int* pos,
-                        const float* w, int tokens, int topk, int H,
-                        hipStream_t stream) {
-  const int threads = 64;
-  const dim3 grid(ceil_div(H / 8, threads), tokens);
-  hipLaunchKernelGGL(moe_combine_kernel, grid, dim3(threads), 0, stream, out,
-                     y, pos, w, topk, H);
-}
-
 // Device-side MoE block alignment in ONE kernel (replaces the ~12-op
 // torch composition in MoEMLP._moe_align: scatter_add histogram,
 // argsort, cumsums, searchsorted, scatters — measured ~6% of 30B MoE
 // GPU time plus a dozen eager launches per layer during prefill).
-// Single workgroup: ≤16K assignments and ≤128 local experts make LDS
+// Single workgroup: ≤16K assignments and ≤1024 local experts make LDS
 // histograms + __syncthreads phases trivial. Within-expert slot order
 // is atomicAdd arrival order (NOT the stable argsort order) — the
 // grouped GEMM computes each row's K-loop identically wherever it sits
@@ -620,8 +584,8 @@ __global__ void moe_align_kernel(
     int* __restrict__ pos,         // [n]  padded slot (-1 = non-local)
     const int n, const int topk, const int e_start, const int e_end,
     const int block_m, const int PM) {
-  const int E = e_end - e_start;  // <= 128 by LDS sizing below
-  __shared__ int cnt[129], pad0[129], tcum[129], off[129];
+  const int E = e_end - e_start;  // <= 1024 by LDS sizing below
+  __shared__ int cnt[1025], pad0[1025], tcum[1025], off[1025];
   const int tid = threadIdx.x, nt = blockDim.x;
   for (int i = tid; i <= E; i += nt) cnt[i] = 0;
   for (int i = tid; i < PM; i += nt) sorted_ids[i] = 0;

@@ -49,6 +49,41 @@ void launch_delta_rule(A*, float*, float*, const A*, const A*, const A*,
                        const float*, float*, const int*, const int*,
                        const int*, int, int, int, int, float, float,
                        hipStream_t);
+template <typename A>
+void launch_layer_norm(A*, const float*, const float*, float, int, int,
+                       hipStream_t);
+template <typename A>
+void launch_gated_residual_layer_norm(float*, const A*, float, const A*, float,
+                                      const A*, int64_t, const float*,
+                                      const float*, A*, float, int, int,
+                                      hipStream_t);
+template <typename A>
+void launch_group_rms_gate(A*, const float*, const A*, int64_t, const float*,
+                           bool, int, int, int, float, bool, hipStream_t);
+template <typename A>
+void launch_paged_cache_write(A*, A*, const A*, int64_t, const A*, int64_t,
+                              const int*, int, int, int, int, int,
+                              hipStream_t);
+template <typename A>
+void launch_decay_linear_attention(float*, float*, float*, const A*, const A*,
+                                   const A*, int64_t, int64_t, int64_t,
+                                   const float*, float*, const int*,
+                                   const int*, const int*, int, int, int, int,
+                                   int, bool, hipStream_t);
+template <typename A>
+void launch_gated_delta_rule(float*, float*, float*, const A*, int64_t,
+                             const float*, const A*, int64_t, const A*,
+                             int64_t, const float*, const float*, float*,
+                             float*, const int*, const int*, const int*,
+                             const int*, int, int, int, int, int, int, int,
+                             hipStream_t);
+size_t talking_window_row_smem(int, int);
+template <typename A>
+void launch_talking_window_rows(A*, const A*, int64_t, const A*, const A*,
+                                const int*, int, const int*, const int*,
+                                const float*, const float*, const float*, int,
+                                int, int, int, int, int, int, float, int,
+                                hipStream_t);
 }  // namespace fi
 
 namespace {
@@ -362,9 +397,266 @@ void delta_rule(at::Tensor out, at::Tensor o_raw, at::Tensor vecs, at::Tensor r,
                         (float)decay_scale, stream()));
 }
 
+
+// ------------------------------------------------------------------------
+// layer-norm / gated-residual stream, decayed linear attention, windowed
+// attention with head mixing, gated delta rule
+
+void layer_norm(at::Tensor out, at::Tensor x, at::Tensor w, double eps) {
+  CHECK_ACT(out);
+  CHECK_F32(x);
+  CHECK_F32(w);
+  TORCH_CHECK(x.dim() == 2 && out.sizes() == x.sizes() && out.is_contiguous());
+  const int T = x.size(0), W = x.size(1);
+  TORCH_CHECK(w.numel() == W);
+  DISPATCH_ACT(out, fi::launch_layer_norm<A>(ptr<A>(out), x.data_ptr<float>(),
+                                             w.data_ptr<float>(), (float)eps,
+                                             T, W, stream()));
+}
+
+void gated_residual_layer_norm(at::Tensor resid, at::Tensor y1, double s1,
+                               c10::optional<at::Tensor> y2, double s2,
+                               at::Tensor gate_lin, at::Tensor gate_bias,
+                               c10::optional<at::Tensor> w_next,
+                               c10::optional<at::Tensor> out, double eps) {
+  CHECK_F32(resid);
+  CHECK_ACT(y1);
+  CHECK_ACT(gate_lin);
+  CHECK_F32(gate_bias);
+  TORCH_CHECK(resid.dim() == 2);
+  const int64_t T = resid.size(0), W = resid.size(1);
+  TORCH_CHECK(y1.sizes() == resid.sizes() && y1.is_contiguous());
+  TORCH_CHECK(gate_lin.scalar_type() == y1.scalar_type());
+  check_rows(gate_lin, T, W, "gate projection");
+  TORCH_CHECK(gate_bias.numel() == W);
+  void* y2p = nullptr;
+  if (y2.has_value()) {
+    TORCH_CHECK(y2->is_cuda() && y2->scalar_type() == y1.scalar_type() &&
+                y2->sizes() == resid.sizes() && y2->is_contiguous());
+    y2p = y2->data_ptr();
+  }
+  TORCH_CHECK(w_next.has_value() == out.has_value());
+  const float* wn = nullptr;
+  void* op = nullptr;
+  if (w_next.has_value()) {
+    CHECK_F32(*w_next);
+    TORCH_CHECK(w_next->numel() == W);
+    TORCH_CHECK(out->is_cuda() && out->scalar_type() == y1.scalar_type() &&
+                out->sizes() == resid.sizes() && out->is_contiguous());
+    wn = w_next->data_ptr<float>();
+    op = out->data_ptr();
+  }
+  DISPATCH_ACT(y1, fi::launch_gated_residual_layer_norm<A>(
+                       resid.data_ptr<float>(), ptr<A>(y1), (float)s1,
+                       reinterpret_cast<const A*>(y2p), (float)s2,
+                       ptr<A>(gate_lin), gate_lin.stride(0),
+                       gate_bias.data_ptr<float>(), wn,
+                       reinterpret_cast<A*>(op), (float)eps, (int)T, (int)W,
+                       stream()));
+}
+
+void group_rms_gate(at::Tensor out, at::Tensor o_raw, at::Tensor glin,
+                    at::Tensor w, int64_t groups, double eps, bool silu) {
+  CHECK_ACT(out);
+  CHECK_F32(o_raw);
+  CHECK_ACT(glin);
+  CHECK_F32(w);
+  TORCH_CHECK(o_raw.dim() == 2 && groups >= 1);
+  const int64_t T = o_raw.size(0), N = o_raw.size(1);
+  TORCH_CHECK(N % groups == 0);
+  const int64_t part = N / groups;
+  TORCH_CHECK(out.sizes() == o_raw.sizes() && out.is_contiguous() &&
+              out.scalar_type() == glin.scalar_type());
+  check_rows(glin, T, N, "gate projection");
+  TORCH_CHECK(w.numel() == N || w.numel() == part,
+              "gain: one per coordinate or one per position in a group");
+  DISPATCH_ACT(out, fi::launch_group_rms_gate<A>(
+                        ptr<A>(out), o_raw.data_ptr<float>(), ptr<A>(glin),
+                        glin.stride(0), w.data_ptr<float>(),
+                        w.numel() != N, (int)T, (int)groups, (int)part,
+                        (float)eps, silu, stream()));
+}
+
+void paged_cache_write(at::Tensor k, at::Tensor v, at::Tensor k_cache,
+                       at::Tensor v_cache, at::Tensor slot_mapping) {
+  CHECK_ACT(k);
+  CHECK_I32(slot_mapping);
+  TORCH_CHECK(k_cache.is_cuda() && v_cache.is_cuda() &&
+              k_cache.is_contiguous() && v_cache.is_contiguous());
+  TORCH_CHECK(k_cache.scalar_type() == k.scalar_type() &&
+              v_cache.scalar_type() == k.scalar_type() &&
+              v.scalar_type() == k.scalar_type() && v.is_cuda());
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 &&
+              k_cache.size(0) == v_cache.size(0) &&
+              k_cache.size(1) == v_cache.size(1) &&
+              k_cache.size(2) == v_cache.size(2));
+  const int64_t T = k.size(0);
+  const int G = k_cache.size(1), bs = k_cache.size(2), D = k_cache.size(3),
+            V = v_cache.size(3);
+  check_rows(k, T, static_cast<int64_t>(G) * D, "keys");
+  check_rows(v, T, static_cast<int64_t>(G) * V, "values");
+  TORCH_CHECK(slot_mapping.numel() == T);
+  DISPATCH_ACT(k, fi::launch_paged_cache_write<A>(
+                      ptr<A>(k_cache), ptr<A>(v_cache), ptr<A>(k), k.stride(0),
+                      ptr<A>(v), v.stride(0), slot_mapping.data_ptr<int>(),
+                      (int)T, G, bs, D, V, stream()));
+}
+
+void check_recurrence_scratch(const at::Tensor& vecs, const at::Tensor& vbuf,
+                              const at::Tensor& o_raw, int64_t T,
+                              int64_t heads, int64_t dim, int64_t vdim) {
+  CHECK_F32(vecs);
+  CHECK_F32(vbuf);
+  CHECK_F32(o_raw);
+  TORCH_CHECK(dim >= 1 && dim <= 256, "recurrence: key size must be <= 256");
+  const int64_t cap = dim <= 64 ? 64 : (dim <= 128 ? 128 : 256);
+  TORCH_CHECK(vecs.numel() == T * heads * 5 * cap,
+              "recurrence scratch must hold [T, heads, 5, ", cap, "]");
+  TORCH_CHECK(vbuf.numel() == T * heads * vdim &&
+              o_raw.numel() == T * heads * vdim);
+}
+
+void decay_linear_attention(at::Tensor o_raw, at::Tensor vecs, at::Tensor vbuf,
+                            at::Tensor q, at::Tensor k, at::Tensor v,
+                            at::Tensor decay, at::Tensor state,
+                            at::Tensor seq_cu, at::Tensor seq_slots,
+                            at::Tensor positions, int64_t heads, int64_t dim,
+                            int64_t vdim, bool silu) {
+  CHECK_ACT(q);
+  const int64_t T = q.size(0);
+  TORCH_CHECK(k.is_cuda() && v.is_cuda() &&
+              k.scalar_type() == q.scalar_type() &&
+              v.scalar_type() == q.scalar_type());
+  check_rows(q, T, heads * dim, "queries");
+  check_rows(k, T, heads * dim, "keys");
+  check_rows(v, T, heads * vdim, "values");
+  check_recurrence_scratch(vecs, vbuf, o_raw, T, heads, dim, vdim);
+  CHECK_F32(decay);
+  CHECK_F32(state);
+  TORCH_CHECK(decay.numel() == heads);
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == heads &&
+              state.size(2) == dim && state.size(3) == vdim);
+  check_groups(seq_cu, seq_slots, positions, T);
+  const int S = seq_slots.numel();
+  DISPATCH_ACT(q, fi::launch_decay_linear_attention<A>(
+                      o_raw.data_ptr<float>(), vecs.data_ptr<float>(),
+                      vbuf.data_ptr<float>(), ptr<A>(q), ptr<A>(k), ptr<A>(v),
+                      q.stride(0), k.stride(0), v.stride(0),
+                      decay.data_ptr<float>(), state.data_ptr<float>(),
+                      seq_cu.data_ptr<int>(), seq_slots.data_ptr<int>(),
+                      positions.data_ptr<int>(), (int)T, S, (int)heads,
+                      (int)dim, (int)vdim, silu, stream()));
+}
+
+void gated_delta_rule(at::Tensor o_raw, at::Tensor vecs, at::Tensor vbuf,
+                      at::Tensor x, at::Tensor conv_w, at::Tensor alin,
+                      at::Tensor blin, at::Tensor a_log, at::Tensor dt_bias,
+                      at::Tensor conv_state, at::Tensor state,
+                      at::Tensor seq_cu, at::Tensor seq_slots,
+                      at::Tensor positions, at::Tensor row_seq, int64_t heads,
+                      int64_t kv_heads, int64_t dim, int64_t vdim) {
+  CHECK_ACT(x);
+  const int64_t T = x.size(0);
+  const int64_t C = 2 * kv_heads * dim + heads * vdim;
+  TORCH_CHECK(kv_heads >= 1 && heads % kv_heads == 0);
+  check_rows(x, T, C, "q|k|v projections");
+  TORCH_CHECK(alin.is_cuda() && blin.is_cuda() &&
+              alin.scalar_type() == x.scalar_type() &&
+              blin.scalar_type() == x.scalar_type());
+  check_rows(alin, T, heads, "decay input");
+  check_rows(blin, T, heads, "write strength input");
+  check_recurrence_scratch(vecs, vbuf, o_raw, T, heads, dim, vdim);
+  CHECK_F32(conv_w);
+  CHECK_F32(a_log);
+  CHECK_F32(dt_bias);
+  CHECK_F32(conv_state);
+  CHECK_F32(state);
+  CHECK_I32(row_seq);
+  TORCH_CHECK(conv_w.dim() == 2 && conv_w.size(0) == C && conv_w.size(1) >= 1);
+  const int taps = conv_w.size(1);
+  TORCH_CHECK(a_log.numel() == heads && dt_bias.numel() == heads);
+  TORCH_CHECK(conv_state.dim() == 3 && conv_state.size(2) == C &&
+              conv_state.size(1) >= taps - 1 &&
+              (taps == 1 || conv_state.size(1) == taps - 1));
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == heads &&
+              state.size(2) == dim && state.size(3) == vdim &&
+              state.size(0) == conv_state.size(0));
+  check_groups(seq_cu, seq_slots, positions, T);
+  TORCH_CHECK(row_seq.numel() == T);
+  const int S = seq_slots.numel();
+  DISPATCH_ACT(x, fi::launch_gated_delta_rule<A>(
+                      o_raw.data_ptr<float>(), vecs.data_ptr<float>(),
+                      vbuf.data_ptr<float>(), ptr<A>(x), x.stride(0),
+                      conv_w.data_ptr<float>(), ptr<A>(alin), alin.stride(0),
+                      ptr<A>(blin), blin.stride(0), a_log.data_ptr<float>(),
+                      dt_bias.data_ptr<float>(), conv_state.data_ptr<float>(),
+                      state.data_ptr<float>(), seq_cu.data_ptr<int>(),
+                      seq_slots.data_ptr<int>(), positions.data_ptr<int>(),
+                      row_seq.data_ptr<int>(), (int)T, S, (int)heads,
+                      (int)kv_heads, (int)dim, (int)vdim, taps, stream()));
+}
+
+void talking_window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
+                              at::Tensor v_cache, at::Tensor seq_bt,
+                              at::Tensor row_seq, at::Tensor positions,
+                              double scale, int64_t window, at::Tensor r1,
+                              at::Tensor r2, at::Tensor talk, int64_t heads) {
+  CHECK_ACT(q);
+  CHECK_I32(seq_bt);
+  CHECK_I32(row_seq);
+  CHECK_I32(positions);
+  CHECK_F32(r1);
+  CHECK_F32(r2);
+  CHECK_F32(talk);
+  TORCH_CHECK(k_cache.is_cuda() && v_cache.is_cuda() &&
+              k_cache.is_contiguous() && v_cache.is_contiguous() &&
+              k_cache.scalar_type() == q.scalar_type() &&
+              v_cache.scalar_type() == q.scalar_type());
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 &&
+              k_cache.size(0) == v_cache.size(0) &&
+              k_cache.size(1) == v_cache.size(1) &&
+              k_cache.size(2) == v_cache.size(2));
+  const int64_t T = q.size(0);
+  const int H = heads, G = k_cache.size(1), bs = k_cache.size(2),
+            D = k_cache.size(3), V = v_cache.size(3);
+  TORCH_CHECK(H >= 1 && G >= 1 && H % G == 0);
+  check_rows(q, T, static_cast<int64_t>(H) * D, "queries");
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() &&
+              out.scalar_type() == q.scalar_type() &&
+              out.numel() == T * H * V);
+  TORCH_CHECK(r1.numel() == H && r2.numel() == H && talk.numel() == H * H);
+  TORCH_CHECK(seq_bt.dim() == 2 && row_seq.numel() == T &&
+              positions.numel() == T);
+  TORCH_CHECK(static_cast<int64_t>(H) * V <= 8192,
+              "windowed attention: heads * vdim must be <= 8192");
+  TORCH_CHECK(fi::talking_window_row_smem(H, D) <= 64 * 1024,
+              "windowed attention: heads * dim too large for one workgroup");
+  DISPATCH_ACT(q, fi::launch_talking_window_rows<A>(
+                      ptr<A>(out), ptr<A>(q), q.stride(0), ptr<A>(k_cache),
+                      ptr<A>(v_cache), seq_bt.data_ptr<int>(),
+                      (int)seq_bt.size(1), row_seq.data_ptr<int>(),
+                      positions.data_ptr<int>(), r1.data_ptr<float>(),
+                      r2.data_ptr<float>(), talk.data_ptr<float>(), 0, (int)T,
+                      H, G, D, V, bs, (float)scale, (int)window, stream()));
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("layer_norm", &layer_norm, "layer norm of an fp32 stream, no bias");
+  m.def("gated_residual_layer_norm", &gated_residual_layer_norm,
+        "fp32 residual += y * sigmoid(gate); optional next layer norm");
+  m.def("group_rms_gate", &group_rms_gate,
+        "grouped unit-RMS of fp32 read-outs with gain and sigmoid/silu gate");
+  m.def("paged_cache_write", &paged_cache_write,
+        "k/v rows into paged caches of separate key and value sizes");
+  m.def("decay_linear_attention", &decay_linear_attention,
+        "linear attention with a scalar decay per head, slot state");
+  m.def("gated_delta_rule", &gated_delta_rule,
+        "gated delta rule behind a short causal convolution, slot state");
+  m.def("talking_window_attention", &talking_window_attention,
+        "windowed softmax attention with log-distance penalty and head "
+        "mixing over the paged cache");
   m.def("scalar_rms_norm", &scalar_rms_norm, "scalar-gain RMS norm");
   m.def("residual_add_scalar_norm", &residual_add_scalar_norm,
         "fp32 residual += norm(y); optional next norm");

@@ -96,13 +96,15 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(
 
 constexpr int kDeltaWaves = 4;   // waves (column tiles) per workgroup
 
+// The state is [dim x vdim] per head (key rows x value columns); v and
+// o_raw rows hold heads*vdim values.
 template <typename A, int DK, int SL, int TB>
 __global__ __launch_bounds__(64 * kDeltaWaves) void delta_rule_wave_kernel(
-    float* __restrict__ o_raw,                  // [T, heads*dim] fp32
+    float* __restrict__ o_raw,                  // [T, heads*vdim] fp32
     const float* __restrict__ vecs,             // [T, heads, 5, DK]
     const A* __restrict__ v, int64_t v_stride, float* __restrict__ state,
     const int* __restrict__ seq_cu, const int* __restrict__ seq_slots,
-    const int* __restrict__ positions, int heads, int dim) {
+    const int* __restrict__ positions, int heads, int dim, int vdim) {
   constexpr int RS = DK / SL;      // rows per lane
   constexpr int R4 = RS / 4;
   constexpr int COLS = 64 / SL;    // columns per wave
@@ -122,8 +124,8 @@ __global__ __launch_bounds__(64 * kDeltaWaves) void delta_rule_wave_kernel(
   const int row0 = seq_cu[s], row1 = seq_cu[s + 1];
   if (row1 <= row0) return;
   const int slot = seq_slots[s];
-  const bool col_ok = c < dim;
-  const int hbase = head * dim;
+  const bool col_ok = c < vdim;
+  const int hbase = head * vdim;
   const int64_t tok_stride = static_cast<int64_t>(heads) * 5 * DK;
   const float* vhead = vecs + static_cast<int64_t>(head) * 5 * DK;
 
@@ -132,12 +134,12 @@ __global__ __launch_bounds__(64 * kDeltaWaves) void delta_rule_wave_kernel(
   for (int j = 0; j < RS; ++j) S[j] = 0.f;
   float* sp = nullptr;
   if (slot >= 0)
-    sp = state + (static_cast<int64_t>(slot) * heads + head) * dim * dim;
+    sp = state + (static_cast<int64_t>(slot) * heads + head) * dim * vdim;
   if (sp != nullptr && positions[row0] > 0 && col_ok) {
 #pragma unroll
     for (int j = 0; j < RS; ++j) {
       const int i = slice * RS + j;
-      if (i < dim) S[j] = sp[static_cast<int64_t>(i) * dim + c];
+      if (i < dim) S[j] = sp[static_cast<int64_t>(i) * vdim + c];
     }
   }
 
@@ -230,7 +232,7 @@ __global__ __launch_bounds__(64 * kDeltaWaves) void delta_rule_wave_kernel(
         }
         const float oc = slice_sum<SL>((o0 + o1) + (o2 + o3));
         if (slice == 0 && col_ok && tt < nt)
-          o_raw[static_cast<int64_t>(tb0 + tt) * heads * dim + hbase + c] = oc;
+          o_raw[static_cast<int64_t>(tb0 + tt) * heads * vdim + hbase + c] = oc;
       }
     }
   }
@@ -238,7 +240,7 @@ __global__ __launch_bounds__(64 * kDeltaWaves) void delta_rule_wave_kernel(
 #pragma unroll
     for (int j = 0; j < RS; ++j) {
       const int i = slice * RS + j;
-      if (i < dim) sp[static_cast<int64_t>(i) * dim + c] = S[j];
+      if (i < dim) sp[static_cast<int64_t>(i) * vdim + c] = S[j];
     }
   }
 }
@@ -274,6 +276,31 @@ inline int delta_row_capacity(int dim) {
   return dim <= 64 ? 64 : (dim <= 128 ? 128 : 256);
 }
 
+// The recurrence alone, on prepared vectors: S <- diag(w) S - (a*u)(u^T S)
+// + k v^T per token, o = S^T r. v rows are of type VT (activations, or
+// fp32 when a preparation kernel has already transformed them).
+template <typename VT>
+void launch_recurrence(float* o_raw, const float* vecs, const VT* v,
+                       int64_t v_stride, float* state, const int* seq_cu,
+                       const int* seq_slots, const int* positions, int S,
+                       int heads, int dim, int vdim, hipStream_t st) {
+  const int DK = delta_row_capacity(dim);
+#define FI_LAUNCH(DKK, SL, TB)                                                 \
+  hipLaunchKernelGGL(                                                          \
+      (delta_rule_wave_kernel<VT, DKK, SL, TB>),                               \
+      dim3(ceil_div(vdim, kDeltaWaves * 64 / SL), heads, S),                   \
+      dim3(64 * kDeltaWaves), 0, st, o_raw, vecs, v, v_stride, state, seq_cu,  \
+      seq_slots, positions, heads, dim, vdim)
+  if (DK == 64) {
+    FI_LAUNCH(64, 8, 8);
+  } else if (DK == 128) {
+    FI_LAUNCH(128, 16, 8);
+  } else {
+    FI_LAUNCH(256, 16, 4);
+  }
+#undef FI_LAUNCH
+}
+
 template <typename A>
 void launch_delta_rule(A* out, float* o_raw, float* vecs, const A* r,
                        const A* k, const A* v, const A* wlin, const A* alin,
@@ -291,22 +318,247 @@ void launch_delta_rule(A* out, float* o_raw, float* vecs, const A* r,
   hipLaunchKernelGGL(delta_prep_kernel<A>, dim3(nblk), dim3(256), 0, st, vecs,
                      r, k, wlin, alin, r_stride, k_stride, w_stride, a_stride,
                      w0, a_bias, T, heads, dim, DK, decay_scale);
-#define FI_LAUNCH(DKK, SL, TB)                                                 \
-  hipLaunchKernelGGL(                                                          \
-      (delta_rule_wave_kernel<A, DKK, SL, TB>),                                \
-      dim3(ceil_div(dim, kDeltaWaves * 64 / SL), heads, S),                    \
-      dim3(64 * kDeltaWaves), 0, st, o_raw, vecs, v, v_stride, state, seq_cu,  \
-      seq_slots, positions, heads, dim)
-  if (DK == 64) {
-    FI_LAUNCH(64, 8, 8);
-  } else if (DK == 128) {
-    FI_LAUNCH(128, 16, 8);
-  } else {
-    FI_LAUNCH(256, 16, 4);
-  }
-#undef FI_LAUNCH
+  launch_recurrence<A>(o_raw, vecs, v, v_stride, state, seq_cu, seq_slots,
+                       positions, S, heads, dim, dim, st);
   hipLaunchKernelGGL(delta_out_gate_kernel<A>, dim3(nblk), dim3(256), 0, st,
                      out, o_raw, glin, g_stride, norm_w, T, heads, dim, eps);
+}
+
+// ---------------------------------------------------------------------
+// Linear attention with one scalar decay per head, as a case of the same
+// recurrence: w = decay_h on every row, nothing removed (a*u = 0),
+// k and r = silu of the key/query projections, v = silu of the value
+// projection (fp32 scratch).
+template <typename A>
+__global__ __launch_bounds__(256) void decay_linear_prep_kernel(
+    float* __restrict__ vecs, float* __restrict__ vbuf,
+    const A* __restrict__ q, const A* __restrict__ k, const A* __restrict__ v,
+    int64_t q_stride, int64_t k_stride, int64_t v_stride,
+    const float* __restrict__ decay, int T, int heads, int dim, int vdim,
+    int DK, bool silu) {
+  const int lane = threadIdx.x % 64;
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / 64;
+  if (item >= static_cast<int64_t>(T) * heads) return;
+  const int t = static_cast<int>(item / heads);
+  const int head = static_cast<int>(item % heads);
+  float* dst = vecs + item * 5 * DK;
+  const float lam = decay[head];
+  for (int i = lane; i < DK; i += 64) {
+    float ww = 1.f, kk = 0.f, rr = 0.f;
+    if (i < dim) {
+      ww = lam;
+      kk = Act<A>::ld(k + t * k_stride + head * dim + i);
+      rr = Act<A>::ld(q + t * q_stride + head * dim + i);
+      if (silu) {
+        kk = kk * sigmoidf_acc(kk);
+        rr = rr * sigmoidf_acc(rr);
+      }
+    }
+    dst[i] = ww;
+    dst[DK + i] = 0.f;
+    dst[2 * DK + i] = 0.f;
+    dst[3 * DK + i] = kk;
+    dst[4 * DK + i] = rr;
+  }
+  for (int c = lane; c < vdim; c += 64) {
+    float vv = Act<A>::ld(v + t * v_stride + head * vdim + c);
+    if (silu) vv = vv * sigmoidf_acc(vv);
+    vbuf[(static_cast<int64_t>(t) * heads + head) * vdim + c] = vv;
+  }
+}
+
+template <typename A>
+void launch_decay_linear_attention(float* o_raw, float* vecs, float* vbuf,
+                                   const A* q, const A* k, const A* v,
+                                   int64_t q_stride, int64_t k_stride,
+                                   int64_t v_stride, const float* decay,
+                                   float* state, const int* seq_cu,
+                                   const int* seq_slots, const int* positions,
+                                   int T, int S, int heads, int dim, int vdim,
+                                   bool silu, hipStream_t st) {
+  if (S == 0 || T == 0) return;
+  const int64_t items = static_cast<int64_t>(T) * heads;
+  const int nblk = static_cast<int>((items + 3) / 4);
+  const int DK = delta_row_capacity(dim);
+  hipLaunchKernelGGL(decay_linear_prep_kernel<A>, dim3(nblk), dim3(256), 0, st,
+                     vecs, vbuf, q, k, v, q_stride, k_stride, v_stride, decay,
+                     T, heads, dim, vdim, DK, silu);
+  launch_recurrence<float>(o_raw, vecs, vbuf,
+                           static_cast<int64_t>(heads) * vdim, state, seq_cu,
+                           seq_slots, positions, S, heads, dim, vdim, st);
+}
+
+// ---------------------------------------------------------------------
+// Gated delta rule behind a short causal convolution, again as a case of
+// the recurrence. With g the head's decay and beta its write strength,
+//   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+// equals S <- g S - (beta g k)(k^T S_old) + k (beta v)^T, i.e. the
+// recurrence with w = g, a*u = beta g k, u = k, v' = beta v, r = q.
+//
+// x rows hold the projections q | k | v (C = 2*kv_heads*dim + heads*vdim
+// channels). y_t[c] = silu(sum_j conv_w[c][j] * x_(t-(taps-1-j))[c]), with
+// inputs from before the step's first row taken from the slot's
+// conv_state [taps-1, C] (oldest first) and zeros before position 0.
+template <typename A>
+struct ConvSrc {
+  const A* x;
+  int64_t x_stride;
+  const float* conv_w;
+  const float* hist;   // slot's conv state or nullptr
+  int taps, C, row0, t, pos;
+  // convolved + silu value of channel c at row t
+  FI_DEV float at(int c) const {
+    float acc = 0.f;
+    for (int j = 0; j < taps; ++j) {
+      const int back = taps - 1 - j;
+      if (back > pos) continue;              // before the sequence start
+      const int src = t - back;
+      float xv;
+      if (src >= row0) {
+        xv = Act<A>::ld(x + src * x_stride + c);
+      } else if (hist != nullptr) {
+        // hist[i] is the input at row0 - (taps-1) + i
+        xv = hist[static_cast<int64_t>(taps - 1 - (row0 - src)) * C + c];
+      } else {
+        xv = 0.f;
+      }
+      acc += conv_w[c * taps + j] * xv;
+    }
+    return acc * sigmoidf_acc(acc);
+  }
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void gated_delta_prep_kernel(
+    float* __restrict__ vecs, float* __restrict__ vbuf,
+    const A* __restrict__ x, int64_t x_stride,
+    const float* __restrict__ conv_w, const A* __restrict__ alin,
+    int64_t a_stride, const A* __restrict__ blin, int64_t b_stride,
+    const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+    const float* __restrict__ conv_state, const int* __restrict__ seq_cu,
+    const int* __restrict__ seq_slots, const int* __restrict__ positions,
+    const int* __restrict__ row_seq, int T, int heads, int kv_heads, int dim,
+    int vdim, int taps, int DK) {
+  const int lane = threadIdx.x % 64;
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / 64;
+  if (item >= static_cast<int64_t>(T) * heads) return;
+  const int t = static_cast<int>(item / heads);
+  const int head = static_cast<int>(item % heads);
+  const int kvh = head / (heads / kv_heads);
+  const int s = row_seq[t];
+  const int slot = seq_slots[s];
+  const int nq = kv_heads * dim;
+  ConvSrc<A> cs;
+  cs.x = x;
+  cs.x_stride = x_stride;
+  cs.conv_w = conv_w;
+  cs.taps = taps;
+  cs.C = 2 * nq + heads * vdim;
+  cs.row0 = seq_cu[s];
+  cs.t = t;
+  cs.pos = positions[t];
+  cs.hist = (slot >= 0 && taps > 1)
+      ? conv_state + static_cast<int64_t>(slot) * (taps - 1) * cs.C
+      : nullptr;
+
+  const float beta = sigmoidf_acc(Act<A>::ld(blin + t * b_stride + head));
+  const float z = Act<A>::ld(alin + t * a_stride + head) + dt_bias[head];
+  const float sp = z > 20.f ? z : log1pf(expf(z));
+  const float g = expf(-expf(a_log[head]) * sp);
+
+  float qsq = 0.f, ksq = 0.f;
+  for (int i = lane; i < dim; i += 64) {
+    const float qv = cs.at(kvh * dim + i);
+    const float kv = cs.at(nq + kvh * dim + i);
+    qsq += qv * qv;
+    ksq += kv * kv;
+  }
+  qsq = wave_reduce_sum(qsq);
+  ksq = wave_reduce_sum(ksq);
+  const float qinv = rsqrtf(qsq + 1e-6f) * rsqrtf(static_cast<float>(dim));
+  const float kinv = rsqrtf(ksq + 1e-6f);
+  float* dst = vecs + item * 5 * DK;
+  for (int i = lane; i < DK; i += 64) {
+    float ww = 1.f, au = 0.f, uu = 0.f, rr = 0.f;
+    if (i < dim) {
+      uu = cs.at(nq + kvh * dim + i) * kinv;
+      rr = cs.at(kvh * dim + i) * qinv;
+      ww = g;
+      au = beta * g * uu;
+    }
+    dst[i] = ww;
+    dst[DK + i] = au;
+    dst[2 * DK + i] = uu;
+    dst[3 * DK + i] = uu;
+    dst[4 * DK + i] = rr;
+  }
+  for (int c = lane; c < vdim; c += 64)
+    vbuf[(static_cast<int64_t>(t) * heads + head) * vdim + c] =
+        beta * cs.at(2 * nq + head * vdim + c);
+}
+
+// New conv state of every sequence group: the last taps-1 inputs, taken
+// from the step's rows or shifted from the old state when the group is
+// shorter; inputs before position 0 are stored as zeros. One thread per
+// (group, channel) reads its old entries before it overwrites them
+// (ascending order: entry j only needs old entries >= j).
+template <typename A>
+__global__ __launch_bounds__(256) void conv_state_update_kernel(
+    float* __restrict__ conv_state, const A* __restrict__ x, int64_t x_stride,
+    const int* __restrict__ seq_cu, const int* __restrict__ seq_slots,
+    const int* __restrict__ positions, int C, int taps) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int slot = seq_slots[s];
+  const int row0 = seq_cu[s], row1 = seq_cu[s + 1];
+  if (slot < 0 || row1 <= row0) return;
+  const int n = row1 - row0;
+  const int pos_end = positions[row0] + n;   // position after the last row
+  float* st = conv_state + static_cast<int64_t>(slot) * (taps - 1) * C + c;
+  for (int j = 0; j < taps - 1; ++j) {
+    // entry j <- input at row index row1 - (taps-1) + j
+    const int back = taps - 1 - j;           // tokens before the end
+    float val;
+    if (back > pos_end) {
+      val = 0.f;                             // before the sequence start
+    } else if (back <= n) {
+      val = Act<A>::ld(x + (row1 - back) * x_stride + c);
+    } else {
+      val = st[static_cast<int64_t>(j + n) * C];   // old entry, j + n > j
+    }
+    st[static_cast<int64_t>(j) * C] = val;
+  }
+}
+
+template <typename A>
+void launch_gated_delta_rule(float* o_raw, float* vecs, float* vbuf,
+                             const A* x, int64_t x_stride, const float* conv_w,
+                             const A* alin, int64_t a_stride, const A* blin,
+                             int64_t b_stride, const float* a_log,
+                             const float* dt_bias, float* conv_state,
+                             float* state, const int* seq_cu,
+                             const int* seq_slots, const int* positions,
+                             const int* row_seq, int T, int S, int heads,
+                             int kv_heads, int dim, int vdim, int taps,
+                             hipStream_t st) {
+  if (S == 0 || T == 0) return;
+  const int64_t items = static_cast<int64_t>(T) * heads;
+  const int nblk = static_cast<int>((items + 3) / 4);
+  const int DK = delta_row_capacity(dim);
+  const int C = 2 * kv_heads * dim + heads * vdim;
+  hipLaunchKernelGGL(gated_delta_prep_kernel<A>, dim3(nblk), dim3(256), 0, st,
+                     vecs, vbuf, x, x_stride, conv_w, alin, a_stride, blin,
+                     b_stride, a_log, dt_bias, conv_state, seq_cu, seq_slots,
+                     positions, row_seq, T, heads, kv_heads, dim, vdim, taps,
+                     DK);
+  if (taps > 1)
+    hipLaunchKernelGGL(conv_state_update_kernel<A>, dim3(ceil_div(C, 256), S),
+                       dim3(256), 0, st, conv_state, x, x_stride, seq_cu,
+                       seq_slots, positions, C, taps);
+  launch_recurrence<float>(o_raw, vecs, vbuf,
+                           static_cast<int64_t>(heads) * vdim, state, seq_cu,
+                           seq_slots, positions, S, heads, dim, vdim, st);
 }
 
 #define FI_INST(A)                                                             \
@@ -315,6 +567,20 @@ void launch_delta_rule(A* out, float* o_raw, float* vecs, const A* r,
       const A*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t,          \
       const float*, const float*, const float*, float*, const int*,            \
       const int*, const int*, int, int, int, int, float, float, hipStream_t);
+FI_INST(float)
+FI_INST(u16)
+#undef FI_INST
+
+#define FI_INST(A)                                                             \
+  template void launch_decay_linear_attention<A>(                              \
+      float*, float*, float*, const A*, const A*, const A*, int64_t, int64_t,  \
+      int64_t, const float*, float*, const int*, const int*, const int*, int,  \
+      int, int, int, int, bool, hipStream_t);                                  \
+  template void launch_gated_delta_rule<A>(                                    \
+      float*, float*, float*, const A*, int64_t, const float*, const A*,       \
+      int64_t, const A*, int64_t, const float*, const float*, float*, float*,  \
+      const int*, const int*, const int*, const int*, int, int, int, int, int, \
+      int, int, hipStream_t);
 FI_INST(float)
 FI_INST(u16)
 #undef FI_INST

@@ -375,3 +375,14 @@ def moe_gemm_fp8(out, a, a_scales, b_packed, b_scales, sorted_ids,
             acc = torch.nn.functional.silu(g) * u
         out[rows] = acc.to(out.dtype)
     return out
+
+
+def moe_route(logits, k: int, score: str, renorm: bool, scale: float):
+    """Router tail: softmax or sigmoid scores, top-k, optional division by
+    the chosen scores' sum (+1e-20), constant factor."""
+    z = logits.float()
+    s = torch.softmax(z, dim=-1) if score == "softmax" else torch.sigmoid(z)
+    topv, topi = s.topk(k, dim=-1)
+    if renorm:
+        topv = topv / (topv.sum(dim=-1, keepdim=True) + 1e-20)
+    return topv * scale, topi.int()

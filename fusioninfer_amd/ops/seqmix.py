@@ -185,3 +185,127 @@ def gelu_tanh_and_mul(gu):
         _native().gelu_tanh_and_mul(out, gu)
         return out
     return ref.gelu_tanh_and_mul(gu)
+
+
+# ------------------------------------------------------------------------
+# layer-norm / gated-residual stream, decayed linear attention, windowed
+# attention with head mixing, gated delta rule
+
+def layer_norm(x, w, eps: float, out_dtype):
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _native().layer_norm(out, x, w, eps)
+        return out
+    return ref.layer_norm(x, w, eps, out_dtype)
+
+
+def gated_residual_layer_norm_(resid, y1, s1: float, y2, s2: float, gate_lin,
+                               gate_bias, w_next, eps: float, out_dtype):
+    """resid (fp32, in place) += (s1*y1 + s2*y2) * sigmoid(gate_lin +
+    gate_bias); returns layer_norm(resid) * w_next (None without w_next).
+    gate_lin may be a column slice of a wider projection output."""
+    if resid.is_cuda:
+        out = None
+        if w_next is not None:
+            out = torch.empty(resid.shape, dtype=out_dtype,
+                              device=resid.device)
+        _native().gated_residual_layer_norm(resid, y1, float(s1), y2,
+                                            float(s2), gate_lin, gate_bias,
+                                            w_next, out, eps)
+        return out
+    return ref.gated_residual_layer_norm_(resid, y1, s1, y2, s2, gate_lin,
+                                          gate_bias, w_next, eps, out_dtype)
+
+
+def _recurrence_scratch(T: int, heads: int, dim: int, device):
+    """fp32 scratch of the recurrence kernel: five vectors per (token,
+    head), padded to the kernel's row capacity for this key size."""
+    if dim > 256:
+        raise ValueError("recurrent mixers support key sizes up to 256")
+    cap = 64 if dim <= 64 else (128 if dim <= 128 else 256)
+    return torch.empty((T, heads, 5, cap), dtype=torch.float32,
+                       device=device)
+
+
+def decay_linear_attention(q, k, v, decay, state, seq_cu, seq_slots,
+                           positions, heads: int, dim: int, vdim: int,
+                           silu: bool = True):
+    """Raw fp32 read-outs [T, heads*vdim] of linear attention with one
+    scalar decay per head; q/k/v may be column slices of one projection
+    output."""
+    if q.is_cuda:
+        T = q.shape[0]
+        o_raw = torch.empty((T, heads * vdim), dtype=torch.float32,
+                            device=q.device)
+        vecs = _recurrence_scratch(T, heads, dim, q.device)
+        vbuf = torch.empty((T, heads * vdim), dtype=torch.float32,
+                           device=q.device)
+        _native().decay_linear_attention(o_raw, vecs, vbuf, q, k, v, decay,
+                                         state, seq_cu, seq_slots, positions,
+                                         heads, dim, vdim, bool(silu))
+        return o_raw
+    return ref.decay_linear_attention(q, k, v, decay, state, seq_cu,
+                                      seq_slots, positions, heads, dim, vdim,
+                                      silu)
+
+
+def group_rms_gate(o_raw, glin, w, groups: int, eps: float, gate: str,
+                   out_dtype):
+    if gate not in ("sigmoid", "silu"):
+        raise ValueError(f"unknown gate {gate!r}")
+    if o_raw.is_cuda:
+        out = torch.empty(o_raw.shape, dtype=out_dtype, device=o_raw.device)
+        _native().group_rms_gate(out, o_raw, glin, w, int(groups), eps,
+                                 gate == "silu")
+        return out
+    return ref.group_rms_gate(o_raw, glin, w, groups, eps, gate, out_dtype)
+
+
+def paged_cache_write_(k, v, k_cache, v_cache, slot_mapping):
+    if k.is_cuda:
+        _native().paged_cache_write(k, v, k_cache, v_cache, slot_mapping)
+        return
+    ref.paged_cache_write_(k, v, k_cache, v_cache, slot_mapping)
+
+
+def talking_window_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
+                             scale: float, window: int, r1, r2, talk,
+                             heads: int, seq_cu=None, tiles=None):
+    """q: [T, heads*dim] (may be a column slice); returns [T, heads, vdim].
+    ``tiles`` as for ranged_paged_attention: the leading row groups that
+    are prompt portions."""
+    T = q.shape[0]
+    dim = q.shape[1] // heads
+    if q.is_cuda:
+        out = torch.empty((T, heads, v_cache.shape[3]), dtype=q.dtype,
+                          device=q.device)
+        _native().talking_window_attention(out, q, k_cache, v_cache, seq_bt,
+                                           row_seq, positions, float(scale),
+                                           int(window), r1, r2, talk,
+                                           int(heads))
+        return out
+    return ref.talking_window_attention(
+        q.reshape(T, heads, dim), k_cache, v_cache, seq_bt, row_seq,
+        positions, scale, window, r1, r2, talk)
+
+
+def gated_delta_rule(x, conv_w, alin, blin, a_log, dt_bias, conv_state,
+                     state, seq_cu, seq_slots, positions, heads: int,
+                     kv_heads: int, dim: int, vdim: int, row_seq=None):
+    """Raw fp32 read-outs [T, heads*vdim] of the gated delta rule behind a
+    short causal convolution; x = q|k|v projections [T, C] (row-strided)."""
+    if x.is_cuda:
+        T = x.shape[0]
+        o_raw = torch.empty((T, heads * vdim), dtype=torch.float32,
+                            device=x.device)
+        vecs = _recurrence_scratch(T, heads, dim, x.device)
+        vbuf = torch.empty((T, heads * vdim), dtype=torch.float32,
+                           device=x.device)
+        _native().gated_delta_rule(o_raw, vecs, vbuf, x, conv_w, alin, blin,
+                                   a_log, dt_bias, conv_state, state, seq_cu,
+                                   seq_slots, positions, row_seq, heads,
+                                   kv_heads, dim, vdim)
+        return o_raw
+    return ref.gated_delta_rule(x, conv_w, alin, blin, a_log, dt_bias,
+                                conv_state, state, seq_cu, seq_slots,
+                                positions, heads, kv_heads, dim, vdim)

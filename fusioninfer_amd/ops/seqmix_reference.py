@@ -206,3 +206,209 @@ def gelu_tanh_and_mul(gu):
     act = 0.5 * g * (1.0 + torch.tanh(
         math.sqrt(2.0 / math.pi) * (g + 0.044715 * g * g * g)))
     return (act * u).to(gu.dtype)
+
+
+# ------------------------------------------------------------------------
+# Layer-norm residual stream with sigmoid-gated sublayer results, linear
+# attention with a scalar decay per head, windowed softmax attention with
+# a log-distance penalty and head mixing, the gated delta rule behind a
+# short causal convolution, grouped unit-RMS output gates.
+
+def layer_norm(x, w, eps: float, out_dtype):
+    """(x - mean) / sqrt(var + eps) * w over the last dim (biased
+    variance, no bias)."""
+    xf = x.float()
+    d = xf - xf.mean(dim=-1, keepdim=True)
+    var = d.pow(2).mean(dim=-1, keepdim=True)
+    return (d * torch.rsqrt(var + eps) * w.float()).to(out_dtype)
+
+
+def gated_residual_layer_norm_(resid, y1, s1: float, y2, s2: float, gate_lin,
+                               gate_bias, w_next, eps: float, out_dtype):
+    """resid += (s1*y1 [+ s2*y2]) * sigmoid(gate_lin + gate_bias) in fp32,
+    in place; optionally returns layer_norm(resid) * w_next."""
+    y = y1.float() * s1
+    if y2 is not None:
+        y = y + y2.float() * s2
+    resid.add_(y * torch.sigmoid(gate_lin.float() + gate_bias.float()))
+    if w_next is None:
+        return None
+    return layer_norm(resid, w_next, eps, out_dtype)
+
+
+def _group_state(state, slot, pos0, shape):
+    if slot < 0 or pos0 == 0:
+        return torch.zeros(shape, dtype=torch.float32)
+    return state[slot].clone()
+
+
+def decay_linear_attention(q, k, v, decay, state, seq_cu, seq_slots,
+                           positions, heads: int, dim: int, vdim: int,
+                           silu: bool = True):
+    """Per head S_t = decay_h * S_(t-1) + k_t v_t^T, o_t = S_t^T q_t with
+    q/k/v passed through silu first when ``silu``. ``state``
+    [slots, heads, dim, vdim] fp32 carries S between steps (zero at
+    position 0). Returns the raw fp32 read-outs [T, heads*vdim]."""
+    T = q.shape[0]
+    act = torch.nn.functional.silu if silu else (lambda z: z)
+    qf = act(q.float()).reshape(T, heads, dim)
+    kf = act(k.float()).reshape(T, heads, dim)
+    vf = act(v.float()).reshape(T, heads, vdim)
+    lam = decay.float().reshape(heads, 1, 1)
+    o = torch.empty(T, heads, vdim, dtype=torch.float32)
+    cu, slots, pos = seq_cu.tolist(), seq_slots.tolist(), positions.tolist()
+    for s in range(len(slots)):
+        a, b = cu[s], cu[s + 1]
+        if b <= a:
+            continue
+        S = _group_state(state, slots[s], pos[a], (heads, dim, vdim))
+        for t in range(a, b):
+            S = lam * S + kf[t][:, :, None] * vf[t][:, None, :]
+            o[t] = torch.einsum("hij,hi->hj", S, qf[t])
+        if slots[s] >= 0:
+            state[slots[s]] = S
+    return o.reshape(T, heads * vdim)
+
+
+def group_rms_gate(o_raw, glin, w, groups: int, eps: float, gate: str,
+                   out_dtype):
+    """Rows of o_raw [T, N] are cut into ``groups`` equal parts, each
+    divided by its root mean square; then times ``w`` ([N], or one part's
+    worth shared by all parts) and sigmoid or silu of glin."""
+    T, N = o_raw.shape
+    part = N // groups
+    o = _rms(o_raw.float().reshape(T, groups, part), eps)
+    wf = w.float()
+    o = o * (wf.reshape(1, 1, part) if wf.numel() == part
+             else wf.reshape(1, groups, part))
+    g = glin.float().reshape(T, groups, part)
+    g = torch.sigmoid(g) if gate == "sigmoid" else \
+        torch.nn.functional.silu(g)
+    return (o * g).reshape(T, N).to(out_dtype)
+
+
+def paged_cache_write_(k, v, k_cache, v_cache, slot_mapping):
+    """Rows of k [T, G*D] / v [T, G*V] into k_cache [B, G, bs, D] /
+    v_cache [B, G, bs, V] at slot_mapping (negative: skipped)."""
+    T = k.shape[0]
+    G, bs = k_cache.shape[1], k_cache.shape[2]
+    slots = slot_mapping.long()
+    ok = slots >= 0
+    blk, off = slots[ok] // bs, slots[ok] % bs
+    k_cache[blk, :, off, :] = k.reshape(T, G, -1)[ok].to(k_cache.dtype)
+    v_cache[blk, :, off, :] = v.reshape(T, G, -1)[ok].to(v_cache.dtype)
+
+
+def talking_window_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
+                             scale: float, window: int, r1, r2, talk):
+    """Softmax attention over the paged keys j of the row's own sequence
+    with 0 <= p - j < window (window <= 0: all j <= p). Per head the raw
+    score is (q.k)*scale - r1_h * ln(1 + r2_h * (p - j)); the heads'
+    scores are then mixed, score_h <- sum_g talk[h, g] score_g, before
+    the softmax. q: [T, H, D]; returns [T, H, V]."""
+    T, H, D = q.shape
+    G, bs = k_cache.shape[1], k_cache.shape[2]
+    rep = H // G
+    out = torch.zeros(T, H, v_cache.shape[3], dtype=torch.float32)
+    pos = positions.tolist()
+    rs = row_seq.tolist()
+    qf = q.float()
+    r1f, r2f, tk = r1.float(), r2.float(), talk.float()
+    t = 0
+    while t < T:
+        s = rs[t]
+        e = t
+        while e + 1 < T and rs[e + 1] == s:
+            e += 1
+        p0, p1 = pos[t], pos[e]
+        lo = max(p0 - window + 1, 0) if window > 0 else 0
+        idx = torch.arange(lo, p1 + 1)
+        blocks = seq_bt[s].long()[idx // bs]
+        kk = k_cache[blocks, :, idx % bs, :].float()
+        vv = v_cache[blocks, :, idx % bs, :].float()
+        kk = kk.repeat_interleave(rep, dim=1)
+        vv = vv.repeat_interleave(rep, dim=1)
+        pr = torch.tensor(pos[t:e + 1])
+        dist = (pr[:, None] - idx[None, :])                  # [rows, keys]
+        vis = dist >= 0
+        if window > 0:
+            vis &= dist < window
+        sc = torch.einsum("ihd,jhd->hij", qf[t:e + 1], kk) * scale
+        dpos = dist.clamp(min=0).float()
+        sc = sc - r1f[:, None, None] * torch.log1p(
+            r2f[:, None, None] * dpos[None])
+        sc = torch.einsum("hg,gij->hij", tk, sc)
+        sc = sc.masked_fill(~vis[None], float("-inf"))
+        w = torch.softmax(sc, dim=-1)
+        out[t:e + 1] = torch.einsum("hij,jhd->ihd", w, vv)
+        t = e + 1
+    return out.to(q.dtype)
+
+
+def gated_delta_rule(x, conv_w, alin, blin, a_log, dt_bias, conv_state,
+                     state, seq_cu, seq_slots, positions, heads: int,
+                     kv_heads: int, dim: int, vdim: int):
+    """Gated delta rule behind a short causal convolution.
+
+    x [T, C] holds the projections q | k | v (kv_heads*dim, kv_heads*dim,
+    heads*vdim channels). Every channel passes a causal convolution over
+    time (conv_w [C, taps], last column = current token, zeros before the
+    sequence start) and silu; q and k become unit vectors per head
+    (x / sqrt(|x|^2 + 1e-6)), q times dim^-0.5. With beta = sigmoid(blin)
+    and g = exp(-exp(a_log) * softplus(alin + dt_bias)), per head
+
+        S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.
+
+    Head h reads q/k head h // (heads // kv_heads). ``conv_state``
+    [slots, taps-1, C] fp32 keeps the last taps-1 inputs, ``state``
+    [slots, heads, dim, vdim] fp32 keeps S. Returns raw fp32 o
+    [T, heads*vdim]."""
+    T, C = x.shape
+    taps = conv_w.shape[1]
+    nq = kv_heads * dim
+    xf = x.float()
+    wf = conv_w.float()
+    rep = heads // kv_heads
+    beta = torch.sigmoid(blin.float())
+    g = torch.exp(-torch.exp(a_log.float())
+                  * torch.nn.functional.softplus(alin.float()
+                                                 + dt_bias.float()))
+    o = torch.empty(T, heads, vdim, dtype=torch.float32)
+    cu, slots, pos = seq_cu.tolist(), seq_slots.tolist(), positions.tolist()
+    for s in range(len(slots)):
+        a, b = cu[s], cu[s + 1]
+        if b <= a:
+            continue
+        slot, p0 = slots[s], pos[a]
+        hist = torch.zeros(taps - 1, C, dtype=torch.float32)
+        if slot >= 0 and p0 > 0 and taps > 1:
+            hist = conv_state[slot].clone()
+            # entries older than the sequence start count as zeros
+            if p0 < taps - 1:
+                hist[: taps - 1 - p0] = 0
+        ext = torch.cat([hist, xf[a:b]], dim=0)              # [taps-1+n, C]
+        y = torch.zeros(b - a, C, dtype=torch.float32)
+        for j in range(taps):
+            y += wf[:, j] * ext[j: j + (b - a)]
+        y = torch.nn.functional.silu(y)
+        if slot >= 0 and taps > 1:
+            conv_state[slot] = ext[-(taps - 1):]
+        qh = y[:, :nq].reshape(-1, kv_heads, dim)
+        kh = y[:, nq:2 * nq].reshape(-1, kv_heads, dim)
+        vh = y[:, 2 * nq:].reshape(-1, heads, vdim)
+        qh = qh * torch.rsqrt(qh.pow(2).sum(-1, keepdim=True) + 1e-6) \
+            * dim ** -0.5
+        kh = kh * torch.rsqrt(kh.pow(2).sum(-1, keepdim=True) + 1e-6)
+        qh = qh.repeat_interleave(rep, dim=1)
+        kh = kh.repeat_interleave(rep, dim=1)
+        S = _group_state(state, slot, p0, (heads, dim, vdim))
+        for i in range(b - a):
+            t = a + i
+            S = g[t][:, None, None] * S
+            u = beta[t][:, None] * (vh[i] - torch.einsum(
+                "hij,hi->hj", S, kh[i]))
+            S = S + kh[i][:, :, None] * u[:, None, :]
+            o[t] = torch.einsum("hij,hi->hj", S, qh[i])
+        if slot >= 0:
+            state[slot] = S
+    return o.reshape(T, heads * vdim)
