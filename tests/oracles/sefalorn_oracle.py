@@ -182,3 +182,14 @@ def forward(tokens, P, cfg, return_layers=False):
     if return_layers:
         return logits, torch.stack(layers)
     return logits
+
+
+def greedy(tokens, P, cfg, n_new):
+    """n_new greedy continuations of a prompt (whole-sequence recompute)."""
+    toks = list(tokens)
+    out = []
+    for _ in range(n_new):
+        nxt = int(forward(toks, P, cfg)[-1].argmax())
+        out.append(nxt)
+        toks.append(nxt)
+    return out
