@@ -72,19 +72,21 @@ def parse_args():
                         "workload mode; headline stays spec-off)")
     p.add_argument("--mixer-compare", action="store_true",
                    help="instead of the serving benchmark: prefill and "
-                        "decode token throughput of the Pinuvik design at "
-                        "real-model layer sizes (random weights) next to "
-                        "the Qwen3-style transformer of the same sizes")
+                        "decode token throughput of the Sefalorn and "
+                        "Pinuvik designs at real-model layer sizes (random "
+                        "weights) next to the Qwen3-style transformer of "
+                        "the same sizes")
     p.add_argument("--mc-sizes", default="2048x16,4096x32",
                    help="WIDTHxHEADS list for --mixer-compare (head dim "
                         "128, kv heads = heads/4, ff = 3*width)")
-    p.add_argument("--mc-archs", default="pinuvik,transformer")
+    p.add_argument("--mc-archs", default="sefalorn,pinuvik,transformer")
     p.add_argument("--mc-layers", type=int, default=4)
     p.add_argument("--mc-prompt", type=int, default=2048)
     p.add_argument("--mc-prefill-seqs", type=int, default=4)
     p.add_argument("--mc-decode-batch", type=int, default=64)
     p.add_argument("--mc-chunk", type=int, default=1024,
-                   help="attention chunk (mask size) of the Pinuvik layers")
+                   help="attention chunk / window (mask size) of the "
+                        "Pinuvik and Sefalorn layers")
     return p.parse_args()
 
 
@@ -101,6 +103,36 @@ def _mixer_compare_config(arch, width, heads, layers, chunk, vocab=32000):
         mc.hidden_size, mc.num_layers = width, layers
         mc.num_heads, mc.num_kv_heads, mc.head_dim = heads, kv, dim
         mc.intermediate_size, mc.vocab_size = ff, vocab
+        return mc
+    if arch == "sefalorn":
+        # lightning and parallel layers in turn; the experts' active size
+        # (top * ff) equals the dense models' ff
+        half = max(heads // 2, 1)
+        moe = {"kind": "moe", "expert": {"ff": ff // 2},
+               "router": {"experts": 8, "top": 2, "scale": 1.0}}
+        lightning = {
+            "type": "lightning",
+            "mixer": {"heads": heads, "dim": dim, "vdim": dim,
+                      "decay": [1.0 - 2.0 ** -(3 + 5 * h / max(heads - 1, 1))
+                                for h in range(heads)]},
+            "mlp": moe}
+        parallel = {
+            "type": "parallel",
+            "mixer": {
+                "left": {"heads": heads, "kv_heads": kv, "dim": dim,
+                         "vdim": dim, "scale": dim ** -0.5,
+                         "mask": {"size": chunk}},
+                "left_scale": 0.5,
+                "right": {"heads": half, "kv_heads": half, "dim": dim,
+                          "vdim": dim, "conv": 4},
+                "right_scale": 0.5},
+            "mlp": moe}
+        raw = {"architecture": "Sefalorn", "vocab": vocab, "width": width,
+               "norm": {"eps": 1e-5}, "logit_scale": 1.0,
+               "layers": [lightning if i % 2 == 0 else parallel
+                          for i in range(layers)]}
+        mc = model_config_from_dict(raw)
+        mc.name = f"sefalorn-{width}x{heads}"
         return mc
     layer = {
         "type": "parallel",

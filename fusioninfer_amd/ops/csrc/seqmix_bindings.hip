@@ -79,6 +79,13 @@ void launch_gated_delta_rule(float*, float*, float*, const A*, int64_t,
                              hipStream_t);
 size_t talking_window_row_smem(int, int);
 template <typename A>
+bool launch_talking_window_tiles(A*, A*, float*, int, const A*, int64_t,
+                                 const A*, const A*, const int*, int,
+                                 const int*, const int*, const float*,
+                                 const float*, const float*, const int*,
+                                 const int*, int, int, int, int, int, int, int,
+                                 float, int, hipStream_t);
+template <typename A>
 void launch_talking_window_rows(A*, const A*, int64_t, const A*, const A*,
                                 const int*, int, const int*, const int*,
                                 const float*, const float*, const float*, int,
@@ -600,7 +607,13 @@ void talking_window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
                               at::Tensor v_cache, at::Tensor seq_bt,
                               at::Tensor row_seq, at::Tensor positions,
                               double scale, int64_t window, at::Tensor r1,
-                              at::Tensor r2, at::Tensor talk, int64_t heads) {
+                              at::Tensor r2, at::Tensor talk, int64_t heads,
+                              c10::optional<at::Tensor> seq_cu,
+                              c10::optional<at::Tensor> tile_seq,
+                              c10::optional<at::Tensor> tile_row0,
+                              int64_t tile_rows,
+                              c10::optional<at::Tensor> folded_q,
+                              c10::optional<at::Tensor> penalty) {
   CHECK_ACT(q);
   CHECK_I32(seq_bt);
   CHECK_I32(row_seq);
@@ -631,13 +644,51 @@ void talking_window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
               "windowed attention: heads * vdim must be <= 8192");
   TORCH_CHECK(fi::talking_window_row_smem(H, D) <= 64 * 1024,
               "windowed attention: heads * dim too large for one workgroup");
+  // the leading tile_rows rows (prompt portions) take the tiled kernel
+  // where the head sizes have a variant; all other rows the row kernel
+  int64_t done = 0;
+  TORCH_CHECK(tile_rows >= 0 && tile_rows <= T);
+  if (tile_rows > 0) {
+    TORCH_CHECK(seq_cu.has_value() && tile_seq.has_value() &&
+                tile_row0.has_value() && folded_q.has_value() &&
+                penalty.has_value());
+    CHECK_I32(*seq_cu);
+    CHECK_I32(*tile_seq);
+    CHECK_I32(*tile_row0);
+    CHECK_F32(*penalty);
+    TORCH_CHECK(tile_seq->numel() == tile_row0->numel());
+    TORCH_CHECK(seq_cu->numel() >= 2);
+    TORCH_CHECK(folded_q->is_cuda() && folded_q->is_contiguous() &&
+                folded_q->scalar_type() == q.scalar_type() &&
+                folded_q->numel() == tile_rows * H * G * D);
+    TORCH_CHECK(penalty->dim() == 2 && penalty->size(0) == H);
+    const int64_t maxd = penalty->size(1);
+    // every distance a row can ask for has an entry
+    TORCH_CHECK(window > 0 ? maxd >= window
+                           : maxd >= seq_bt.size(1) * bs,
+                "penalty table too short");
+    bool ok = false;
+    DISPATCH_ACT(q, ok = fi::launch_talking_window_tiles<A>(
+                        ptr<A>(out), ptr<A>(*folded_q),
+                        penalty->data_ptr<float>(), (int)maxd, ptr<A>(q),
+                        q.stride(0), ptr<A>(k_cache), ptr<A>(v_cache),
+                        seq_bt.data_ptr<int>(), (int)seq_bt.size(1),
+                        seq_cu->data_ptr<int>(), positions.data_ptr<int>(),
+                        r1.data_ptr<float>(), r2.data_ptr<float>(),
+                        talk.data_ptr<float>(), tile_seq->data_ptr<int>(),
+                        tile_row0->data_ptr<int>(), (int)tile_seq->numel(),
+                        (int)tile_rows, H, G, D, V, bs, (float)scale,
+                        (int)window, stream()));
+    if (ok) done = tile_rows;
+  }
   DISPATCH_ACT(q, fi::launch_talking_window_rows<A>(
                       ptr<A>(out), ptr<A>(q), q.stride(0), ptr<A>(k_cache),
                       ptr<A>(v_cache), seq_bt.data_ptr<int>(),
                       (int)seq_bt.size(1), row_seq.data_ptr<int>(),
                       positions.data_ptr<int>(), r1.data_ptr<float>(),
-                      r2.data_ptr<float>(), talk.data_ptr<float>(), 0, (int)T,
-                      H, G, D, V, bs, (float)scale, (int)window, stream()));
+                      r2.data_ptr<float>(), talk.data_ptr<float>(), (int)done,
+                      (int)(T - done), H, G, D, V, bs, (float)scale,
+                      (int)window, stream()));
 }
 
 }  // namespace

@@ -13,6 +13,22 @@
 // query rows (tile kernel). Scores, the mixing, the softmax and the
 // weighted sum are fp32; keys/values are read in the cache's type.
 //
+// Tile kernel (prompt portions): the mixing is linear in the queries, so
+// it is folded into them first,
+//
+//   mixed_h[j] = scale * sum_kv (q'_(h,kv) . k_kv[j]) - pen'_h(p - j),
+//   q'_(h,kv)  = sum_{g in kv} talk[h][g] q_g          (fp32 sum)
+//   pen'_h(d)  = sum_g talk[h][g] r1_g ln(1 + r2_g d)   (fp32 table)
+//
+// which is ordinary attention of head h with one query segment per kv
+// head. A 4-wave workgroup takes 128 consecutive rows of one (sequence,
+// head), 32 per wave, walks the key range in LDS-staged tiles, and for
+// every tile accumulates S^T = sum_kv K_kv Q'_kv^T on the matrix cores
+// (bf16 16x16x16, or true-fp32 16x16x4), one kv head's key tile in LDS at
+// a time; the value tile of the head's own kv head is staged with the
+// first segment. Softmax statistics stay fp32 per lane (one query per
+// lane column). O^T += V^T P^T as in the shared-key/value tile kernel.
+//
 // Row kernel (decode rows, and any row when no tile table is given):
 // 256 threads per row, key tiles of KT keys, five phases per tile: raw
 // scores -> LDS, mixing -> LDS, per-head running maximum, exponentials
@@ -20,6 +36,8 @@
 // (head, value column) outputs in registers.
 
 #include <math.h>
+
+#include <type_traits>
 
 #include "seqmix.h"
 
@@ -150,6 +168,315 @@ __global__ __launch_bounds__(256) void talking_window_row_kernel(
   }
 }
 
+
+typedef __attribute__((ext_vector_type(4))) short short4v;
+typedef __attribute__((ext_vector_type(4))) float floatx4;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+
+constexpr int kQSets = 2;               // 16-row query sets per wave
+constexpr int kTileRows = 64 * kQSets;  // q rows per workgroup (4 waves)
+
+// q' [T, H, G, D] = sum over the q heads g of kv head kv of talk[h][g] q_g
+template <typename A>
+__global__ __launch_bounds__(256) void talking_fold_queries_kernel(
+    A* __restrict__ qf, const A* __restrict__ q, int64_t q_stride,
+    const float* __restrict__ talk, int H, int G, int D) {
+  const int64_t t = blockIdx.x;
+  const int rep = H / G;
+  const int n = H * G * D;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const int d = i % D;
+    const int kv = (i / D) % G;
+    const int h = i / (D * G);
+    float acc = 0.f;
+    for (int r = 0; r < rep; ++r) {
+      const int g = kv * rep + r;
+      acc += talk[h * H + g] * Act<A>::ld(q + t * q_stride + g * D + d);
+    }
+    Act<A>::st(qf + t * n + i, acc);
+  }
+}
+
+// pen' [H, maxd]
+__global__ __launch_bounds__(256) void talking_penalty_table_kernel(
+    float* __restrict__ pen, const float* __restrict__ r1,
+    const float* __restrict__ r2, const float* __restrict__ talk, int H,
+    int maxd) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= H * maxd) return;
+  const int h = i / maxd;
+  const float d = static_cast<float>(i % maxd);
+  float acc = 0.f;
+  for (int g = 0; g < H; ++g)
+    acc += talk[h * H + g] * r1[g] * log1pf(r2[g] * d);
+  pen[i] = acc;
+}
+
+template <typename A, int D, int DV, int BN>
+__global__ __launch_bounds__(256) void talking_window_tile_kernel(
+    A* __restrict__ out,                 // [T, H, DV]
+    const A* __restrict__ qf,            // [T, H, G, D] folded queries
+    const A* __restrict__ k_cache,       // [B, G, bs, D]
+    const A* __restrict__ v_cache,       // [B, G, bs, DV]
+    const float* __restrict__ pen, int maxd,   // [H, maxd]
+    const int* __restrict__ seq_bt, int bt_stride,
+    const int* __restrict__ seq_cu, const int* __restrict__ positions,
+    const int* __restrict__ tile_seq, const int* __restrict__ tile_row0, int H,
+    int G, int block_size, float scale, int window) {
+  constexpr bool BF = std::is_same<A, u16>::value;
+  constexpr int QS = kQSets;
+  constexpr int VEC = BF ? 8 : 4;               // elements per 16-byte load
+  constexpr int KP = D + (BF ? 8 : 4);          // K tile [BN][KP]
+  constexpr int VP = BF ? BN + 8 : DV + 4;      // bf16: V^T [DV][VP]; fp32: V [BN][VP]
+  constexpr int NB = BN / 16;
+  constexpr int DB = D / 16;
+  constexpr int VB = DV / 16;
+  __shared__ __attribute__((aligned(16))) A k_lds[BN * KP];
+  __shared__ __attribute__((aligned(16))) A v_lds[BF ? DV * VP : BN * VP];
+
+  const int tid = threadIdx.x;
+  const int wave = tid / 64, lane = tid % 64;
+  const int g4 = lane / 16, c16 = lane % 16;
+  const int h = blockIdx.y;
+  const int gv = h / (H / G);                   // the head's value kv head
+  const int s = tile_seq[blockIdx.x];
+  const int row_first = seq_cu[s] + tile_row0[blockIdx.x];
+  const int nrows = min(kTileRows, seq_cu[s + 1] - row_first);
+  const int* bt = seq_bt + static_cast<int64_t>(s) * bt_stride;
+  const float* pen_h = pen + static_cast<int64_t>(h) * maxd;
+
+  auto range_lo = [&](int p) { return window > 0 ? max(p - window + 1, 0) : 0; };
+  const int p_first = positions[row_first];
+  const int kv_lo = range_lo(p_first);
+  const int kv_hi = p_first + nrows - 1;   // positions in a group ascend by 1
+
+  // this lane's queries: column c16 of each of the wave's 16-row sets
+  int my_row[QS], my_pos[QS], my_lo[QS];
+  bool row_ok[QS];
+  const A* my_q[QS];
+#pragma unroll
+  for (int qs = 0; qs < QS; ++qs) {
+    my_row[qs] = (wave * QS + qs) * 16 + c16;
+    row_ok[qs] = my_row[qs] < nrows;
+    my_pos[qs] = row_ok[qs] ? p_first + my_row[qs] : -1;
+    my_lo[qs] = row_ok[qs] ? range_lo(my_pos[qs]) : 0;
+    my_q[qs] = qf + (static_cast<int64_t>(row_first +
+                                          (row_ok[qs] ? my_row[qs] : 0)) * H +
+                     h) * G * D;
+  }
+
+  floatx4 o[QS][VB];
+  float m[QS], l[QS];
+#pragma unroll
+  for (int qs = 0; qs < QS; ++qs) {
+    m[qs] = -INFINITY;
+    l[qs] = 0.f;
+#pragma unroll
+    for (int vb = 0; vb < VB; ++vb) o[qs][vb] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int j0 = kv_lo; j0 <= kv_hi; j0 += BN) {
+    floatx4 sacc[QS][NB];
+#pragma unroll
+    for (int qs = 0; qs < QS; ++qs)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) sacc[qs][nb] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    for (int kv = 0; kv < G; ++kv) {
+      // ---- stage this kv head's K tile (and, once, the V tile) ----
+      constexpr int KPR = D / VEC;               // vectors per key row
+      constexpr int VPR = DV / VEC;
+      for (int vid = tid; vid < BN * KPR; vid += 256) {
+        const int key_l = vid / KPR, dv = vid % KPR;
+        const int key = j0 + key_l;
+        u32x4 k4 = {0u, 0u, 0u, 0u};
+        if (key <= kv_hi) {
+          const int64_t off =
+              ((static_cast<int64_t>(bt[key / block_size]) * G + kv) *
+                   block_size + key % block_size) * D + dv * VEC;
+          k4 = *reinterpret_cast<const u32x4*>(k_cache + off);
+        }
+        *reinterpret_cast<u32x4*>(k_lds + key_l * KP + dv * VEC) = k4;
+      }
+      if (kv == 0) {
+        if constexpr (BF) {
+          // two adjacent keys per thread: the transposed V tile is written
+          // with 4-byte stores (one (key, key+1) pair per value column)
+          for (int pid = tid; pid < (BN / 2) * VPR; pid += 256) {
+            const int kp = pid / VPR, dv = pid % VPR;
+            u32x4 v4[2];
+#pragma unroll
+            for (int e2 = 0; e2 < 2; ++e2) {
+              const int key = j0 + 2 * kp + e2;
+              v4[e2] = u32x4{0u, 0u, 0u, 0u};
+              if (key <= kv_hi) {
+                const int64_t off =
+                    ((static_cast<int64_t>(bt[key / block_size]) * G + gv) *
+                         block_size + key % block_size) * DV + dv * VEC;
+                v4[e2] = *reinterpret_cast<const u32x4*>(v_cache + off);
+              }
+            }
+            const u16* va = reinterpret_cast<const u16*>(&v4[0]);
+            const u16* vb = reinterpret_cast<const u16*>(&v4[1]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              *reinterpret_cast<u32*>(v_lds + (dv * 8 + e) * VP + 2 * kp) =
+                  static_cast<u32>(va[e]) | (static_cast<u32>(vb[e]) << 16);
+          }
+        } else {
+          for (int vid = tid; vid < BN * VPR; vid += 256) {
+            const int key_l = vid / VPR, dv = vid % VPR;
+            const int key = j0 + key_l;
+            u32x4 vv4 = {0u, 0u, 0u, 0u};
+            if (key <= kv_hi) {
+              const int64_t off =
+                  ((static_cast<int64_t>(bt[key / block_size]) * G + gv) *
+                       block_size + key % block_size) * DV + dv * VEC;
+              vv4 = *reinterpret_cast<const u32x4*>(v_cache + off);
+            }
+            *reinterpret_cast<u32x4*>(v_lds + key_l * VP + dv * VEC) = vv4;
+          }
+        }
+      }
+      __syncthreads();
+
+      // ---- S^T += K_kv Q'_kv^T ----
+      if constexpr (BF) {
+        short4v qfr[QS][DB];
+#pragma unroll
+        for (int qs = 0; qs < QS; ++qs)
+#pragma unroll
+          for (int kk = 0; kk < DB; ++kk)
+            qfr[qs][kk] = row_ok[qs]
+                ? *reinterpret_cast<const short4v*>(my_q[qs] + kv * D +
+                                                    16 * kk + 4 * g4)
+                : short4v{0, 0, 0, 0};
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const A* kr = k_lds + (nb * 16 + c16) * KP;
+#pragma unroll
+          for (int kk = 0; kk < DB; ++kk) {
+            const short4v a =
+                *reinterpret_cast<const short4v*>(kr + 16 * kk + 4 * g4);
+#pragma unroll
+            for (int qs = 0; qs < QS; ++qs)
+              sacc[qs][nb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+                  a, qfr[qs][kk], sacc[qs][nb], 0, 0, 0);
+          }
+        }
+      } else {
+#pragma unroll 4
+        for (int kk = 0; kk < D / 4; ++kk) {
+          float qv[QS];
+#pragma unroll
+          for (int qs = 0; qs < QS; ++qs)
+            qv[qs] = row_ok[qs] ? my_q[qs][kv * D + 4 * kk + g4] : 0.f;
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            const float a = k_lds[(nb * 16 + c16) * KP + 4 * kk + g4];
+#pragma unroll
+            for (int qs = 0; qs < QS; ++qs)
+              sacc[qs][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                  a, qv[qs], sacc[qs][nb], 0, 0, 0);
+          }
+        }
+      }
+      // the next segment overwrites the K tile
+      if (kv + 1 < G) __syncthreads();
+    }
+
+    // ---- scale, distance penalty, mask, online softmax ----
+    float sv[QS][NB][4];
+#pragma unroll
+    for (int qs = 0; qs < QS; ++qs) {
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = j0 + nb * 16 + 4 * g4 + i;
+          const bool vis = key <= my_pos[qs] && key >= my_lo[qs];
+          float x = -INFINITY;
+          if (vis) x = sacc[qs][nb][i] * scale - pen_h[my_pos[qs] - key];
+          sv[qs][nb][i] = x;
+          tmax = fmaxf(tmax, x);
+        }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m[qs], tmax);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float corr = expf(m[qs] - m_safe);     // m = -inf -> 0
+      float psum = 0.f;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          sv[qs][nb][i] = expf(sv[qs][nb][i] - m_safe);  // masked -> 0
+          psum += sv[qs][nb][i];
+        }
+      psum += __shfl_xor(psum, 16, 64);
+      psum += __shfl_xor(psum, 32, 64);
+      l[qs] = l[qs] * corr + psum;
+      m[qs] = m_new;
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[qs][vb][i] *= corr;
+    }
+
+    // ---- O^T += V^T P^T: every V fragment feeds QS MFMAs ----
+    if constexpr (BF) {
+      short4v pf[QS][NB];
+#pragma unroll
+      for (int qs = 0; qs < QS; ++qs)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            pf[qs][nb][i] = static_cast<short>(f32_to_bf16(sv[qs][nb][i]));
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb) {
+        const A* vr = v_lds + (vb * 16 + c16) * VP;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const short4v a =
+              *reinterpret_cast<const short4v*>(vr + nb * 16 + 4 * g4);
+#pragma unroll
+          for (int qs = 0; qs < QS; ++qs)
+            o[qs][vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+                a, pf[qs][nb], o[qs][vb], 0, 0, 0);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float a = v_lds[(nb * 16 + 4 * g4 + i) * VP + vb * 16 + c16];
+#pragma unroll
+            for (int qs = 0; qs < QS; ++qs)
+              o[qs][vb] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                  a, sv[qs][nb][i], o[qs][vb], 0, 0, 0);
+          }
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int qs = 0; qs < QS; ++qs) {
+    if (!row_ok[qs]) continue;
+    const float inv_l = 1.0f / l[qs];
+    A* op = out + (static_cast<int64_t>(row_first + my_row[qs]) * H + h) * DV;
+#pragma unroll
+    for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        Act<A>::st(op + vb * 16 + 4 * g4 + i, o[qs][vb][i] * inv_l);
+  }
+}
+
 }  // namespace
 
 size_t talking_window_row_smem(int H, int D) {
@@ -188,7 +515,61 @@ void launch_talking_window_rows(A* out, const A* q, int64_t q_stride,
 #undef FI_LAUNCH
 }
 
+
+// Prompt-portion rows [0, tile_rows) through the folded tile kernel.
+// Returns false when the head sizes have no tiled variant (the caller
+// then runs those rows through the row kernel).
+template <typename A>
+bool launch_talking_window_tiles(A* out, A* qf, float* pen, int maxd,
+                                 const A* q, int64_t q_stride,
+                                 const A* k_cache, const A* v_cache,
+                                 const int* seq_bt, int bt_width,
+                                 const int* seq_cu, const int* positions,
+                                 const float* r1, const float* r2,
+                                 const float* talk, const int* tile_seq,
+                                 const int* tile_row0, int num_tiles,
+                                 int tile_rows, int H, int G, int D, int V,
+                                 int bs, float scale, int window,
+                                 hipStream_t st) {
+  constexpr bool BF = std::is_same<A, u16>::value;
+  if (num_tiles == 0 || tile_rows == 0) return true;
+  const bool fits = (D == 32 || D == 64 || D == 128) &&
+                    (V == 32 || V == 64 || V == 128);
+  if (!fits) return false;
+  hipLaunchKernelGGL(talking_fold_queries_kernel<A>, dim3(tile_rows),
+                     dim3(256), 0, st, qf, q, q_stride, talk, H, G, D);
+  hipLaunchKernelGGL(talking_penalty_table_kernel,
+                     dim3(ceil_div(H * maxd, 256)), dim3(256), 0, st, pen, r1,
+                     r2, talk, H, maxd);
+  dim3 grid(num_tiles, H);
+#define FI_TILE(DD, VV, BNB, BNF)                                             \
+  if (D == DD && V == VV) {                                                   \
+    hipLaunchKernelGGL(                                                       \
+        (talking_window_tile_kernel<A, DD, VV, (BF ? BNB : BNF)>), grid,      \
+        dim3(256), 0, st, out, qf, k_cache, v_cache, pen, maxd, seq_bt,       \
+        bt_width, seq_cu, positions, tile_seq, tile_row0, H, G, bs, scale,    \
+        window);                                                              \
+    return true;                                                              \
+  }
+  FI_TILE(32, 32, 64, 64)
+  FI_TILE(32, 64, 64, 64)
+  FI_TILE(32, 128, 64, 32)
+  FI_TILE(64, 32, 64, 64)
+  FI_TILE(64, 64, 64, 64)
+  FI_TILE(64, 128, 64, 32)
+  FI_TILE(128, 32, 64, 32)
+  FI_TILE(128, 64, 64, 32)
+  FI_TILE(128, 128, 64, 32)
+#undef FI_TILE
+  return false;
+}
+
 #define FI_INST(A)                                                            \
+  template bool launch_talking_window_tiles<A>(                               \
+      A*, A*, float*, int, const A*, int64_t, const A*, const A*, const int*, \
+      int, const int*, const int*, const float*, const float*, const float*,  \
+      const int*, const int*, int, int, int, int, int, int, int, float, int,  \
+      hipStream_t);                                                           \
   template void launch_talking_window_rows<A>(                                \
       A*, const A*, int64_t, const A*, const A*, const int*, int, const int*, \
       const int*, const float*, const float*, const float*, int, int, int,    \

@@ -279,10 +279,25 @@ def talking_window_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
     if q.is_cuda:
         out = torch.empty((T, heads, v_cache.shape[3]), dtype=q.dtype,
                           device=q.device)
+        tile_seq = tile_row0 = folded = pen = None
+        tile_rows = 0
+        if tiles is not None and seq_cu is not None and tiles[2] > 0:
+            tile_seq, tile_row0, tile_rows = tiles
+            # scratch of the tiled kernel: queries with the head mixing
+            # folded in (one segment per kv head) and the mixed distance
+            # penalty for every distance a row can reach
+            G, bs = k_cache.shape[1], k_cache.shape[2]
+            folded = torch.empty((tile_rows, heads, G, dim), dtype=q.dtype,
+                                 device=q.device)
+            maxd = int(window) if window > 0 else seq_bt.shape[1] * bs
+            pen = torch.empty((heads, maxd), dtype=torch.float32,
+                              device=q.device)
         _native().talking_window_attention(out, q, k_cache, v_cache, seq_bt,
                                            row_seq, positions, float(scale),
                                            int(window), r1, r2, talk,
-                                           int(heads))
+                                           int(heads), seq_cu, tile_seq,
+                                           tile_row0, int(tile_rows), folded,
+                                           pen)
         return out
     return ref.talking_window_attention(
         q.reshape(T, heads, dim), k_cache, v_cache, seq_bt, row_seq,

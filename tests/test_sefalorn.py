@@ -326,6 +326,31 @@ def test_window_edge_one_key_in_or_out(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("H,G,dim,vdim,window", [
+    (4, 2, 32, 64, 50), (2, 1, 64, 32, 200), (4, 4, 128, 128, 37),
+    (6, 3, 64, 128, 129)])
+def test_window_attention_tiled_sizes(device, H, G, dim, vdim, window):
+    """Head sizes that take the matrix-core tile kernel on the GPU, rows
+    beyond one 128-row tile, windows that end inside key tiles."""
+    got, want = _window_case(device, H, G, dim, vdim, window, T=300,
+                             cut=171, decode_tail=3)
+    assert (got - want).abs().max() < 5e-5
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_window_edge_in_tiled_prompt_portions(device):
+    """window = 130 over 128-row tiles and 64-key tiles: the key at
+    distance 129 is seen, the one at distance 130 is not, for rows in the
+    first and the second portion."""
+    for boost in [(260, 131), (260, 130), (150, 21), (150, 20), (299, 170),
+                  (299, 169)]:
+        got, want = _window_case(device, 2, 1, 32, 32, 130, T=300,
+                                 boost=boost, seed=boost[0] + boost[1],
+                                 cut=171)
+        assert (got - want).abs().max() < 5e-5, boost
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_window_spanning_many_pages(device):
     got, want = _window_case(device, 4, 2, 16, 24, 150, T=330,
                              boost=(329, 180), seed=5, cut=301)
