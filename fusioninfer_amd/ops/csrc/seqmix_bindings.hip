@@ -78,6 +78,8 @@ void launch_gated_delta_rule(float*, float*, float*, const A*, int64_t,
                              const int*, int, int, int, int, int, int, int,
                              hipStream_t);
 size_t talking_window_row_smem(int, int);
+bool talking_window_fast_fits(int, int, int, int);
+int talking_window_fast_splits(int);
 template <typename A>
 bool launch_talking_window_tiles(A*, A*, float*, int, const A*, int64_t,
                                  const A*, const A*, const int*, int,
@@ -90,7 +92,7 @@ void launch_talking_window_rows(A*, const A*, int64_t, const A*, const A*,
                                 const int*, int, const int*, const int*,
                                 const float*, const float*, const float*, int,
                                 int, int, int, int, int, int, float, int,
-                                hipStream_t);
+                                float*, float*, int, hipStream_t);
 }  // namespace fi
 
 namespace {
@@ -613,7 +615,9 @@ void talking_window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
                               c10::optional<at::Tensor> tile_row0,
                               int64_t tile_rows,
                               c10::optional<at::Tensor> folded_q,
-                              c10::optional<at::Tensor> penalty) {
+                              c10::optional<at::Tensor> penalty,
+                              c10::optional<at::Tensor> part_ml,
+                              c10::optional<at::Tensor> part_o) {
   CHECK_ACT(q);
   CHECK_I32(seq_bt);
   CHECK_I32(row_seq);
@@ -681,14 +685,35 @@ void talking_window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
                         (int)window, stream()));
     if (ok) done = tile_rows;
   }
+  // remaining rows: partial results per 256-key pass when the
+  // thread-per-key kernel fits and scratch was handed in
+  float* pml = nullptr;
+  float* pob = nullptr;
+  int nsplit = 1;
+  const int64_t rest = T - done;
+  if (rest > 0 && part_ml.has_value() && part_o.has_value() &&
+      fi::talking_window_fast_fits(H, G, D, V)) {
+    CHECK_F32(*part_ml);
+    CHECK_F32(*part_o);
+    const int64_t max_keys = window > 0 ? window : seq_bt.size(1) * bs;
+    nsplit = fi::talking_window_fast_splits((int)max_keys);
+    // scratch sized for the decoded rows only: when prompt rows come here
+    // too (no tiled variant for these head sizes) all rows take the
+    // one-workgroup-per-row kernel
+    if (part_ml->numel() >= rest * nsplit * 2 * H &&
+        part_o->numel() >= rest * nsplit * H * V) {
+      pml = part_ml->data_ptr<float>();
+      pob = part_o->data_ptr<float>();
+    }
+  }
   DISPATCH_ACT(q, fi::launch_talking_window_rows<A>(
                       ptr<A>(out), ptr<A>(q), q.stride(0), ptr<A>(k_cache),
                       ptr<A>(v_cache), seq_bt.data_ptr<int>(),
                       (int)seq_bt.size(1), row_seq.data_ptr<int>(),
                       positions.data_ptr<int>(), r1.data_ptr<float>(),
                       r2.data_ptr<float>(), talk.data_ptr<float>(), (int)done,
-                      (int)(T - done), H, G, D, V, bs, (float)scale,
-                      (int)window, stream()));
+                      (int)rest, H, G, D, V, bs, (float)scale, (int)window,
+                      pml, pob, nsplit, stream()));
 }
 
 }  // namespace
@@ -705,6 +730,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "linear attention with a scalar decay per head, slot state");
   m.def("gated_delta_rule", &gated_delta_rule,
         "gated delta rule behind a short causal convolution, slot state");
+  m.def("talking_window_splits", &fi::talking_window_fast_splits,
+        "key passes per row of the thread-per-key windowed attention");
   m.def("talking_window_attention", &talking_window_attention,
         "windowed softmax attention with log-distance penalty and head "
         "mixing over the paged cache");

@@ -169,6 +169,193 @@ __global__ __launch_bounds__(256) void talking_window_row_kernel(
 }
 
 
+
+// Row kernel, thread-per-key form (decode rows when the sizes allow 4-wide
+// accesses): 256 keys per pass, one per thread. A thread reads its key's
+// rows of all kv heads once (vector loads), forms the raw scores of all
+// heads against the query held in LDS (broadcast reads), mixes them in
+// registers, and the block then takes per-head maxima and sums across
+// threads (wave shuffles + one LDS hop). For the weighted value sum the
+// threads switch to owning (head, 4 value columns) outputs and walk the
+// pass's weights in LDS.
+constexpr int kFastKT = 256;
+constexpr int kFastMaxRep = 8;
+constexpr int kFastItems = 4;      // (head, 4 columns) outputs per thread
+
+template <typename A, int MAXH>
+__global__ __launch_bounds__(256) void talking_window_row_fast_kernel(
+    float* __restrict__ part_ml,         // [rows, nsplit, 2, H] max, sum
+    float* __restrict__ part_o,          // [rows, nsplit, H*V]
+    const A* __restrict__ q, int64_t q_stride,
+    const A* __restrict__ k_cache, const A* __restrict__ v_cache,
+    const int* __restrict__ seq_bt, int bt_width,
+    const int* __restrict__ row_seq, const int* __restrict__ positions,
+    const float* __restrict__ r1, const float* __restrict__ r2,
+    const float* __restrict__ talk, int row_begin, int H, int G, int D, int V,
+    int bs, float scale, int window) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  float* qs = smem;                      // [H*D]
+  float* pbuf = qs + H * D;              // [H][KT] weights of this pass
+  float* tk = pbuf + H * kFastKT;        // [H][H]
+  float* wred = tk + H * H;              // [4][H] per-wave partials
+
+  const int t = row_begin + blockIdx.x;
+  const int split = blockIdx.y, nsplit = gridDim.y;
+  const int tid = threadIdx.x;
+  const int wave = tid / 64, lane = tid % 64;
+  const int s = row_seq[t];
+  const int p = positions[t];
+  const int lo = window > 0 ? max(p - window + 1, 0) : 0;
+  const int* bt = seq_bt + static_cast<int64_t>(s) * bt_width;
+  const int rep = H / G;
+  const int nitems = H * V / 4;
+  const int64_t pslot = static_cast<int64_t>(blockIdx.x) * nsplit + split;
+  float* pml = part_ml + pslot * 2 * H;
+  float* po = part_o + pslot * H * V;
+
+  // this workgroup's 256 keys
+  const int j0 = lo + split * kFastKT;
+  if (j0 > p) {                          // nothing to see: an empty partial
+    if (tid < H) {
+      pml[tid] = -INFINITY;
+      pml[H + tid] = 0.f;
+    }
+    return;
+  }
+  for (int i = tid; i < H * D; i += 256)
+    qs[i] = Act<A>::ld(q + t * q_stride + i);
+  for (int i = tid; i < H * H; i += 256) tk[i] = talk[i];
+  __syncthreads();
+
+  const int j = j0 + tid;
+  const bool live = j <= p;
+  float raw[MAXH];
+#pragma unroll
+  for (int g = 0; g < MAXH; ++g) raw[g] = 0.f;
+  if (live) {
+    const int64_t blk = bt[j / bs];
+    const float dist = static_cast<float>(p - j);
+    for (int kv = 0; kv < G; ++kv) {
+      const A* kr = k_cache + ((blk * G + kv) * bs + j % bs) * D;
+      float part[kFastMaxRep];
+#pragma unroll
+      for (int r = 0; r < kFastMaxRep; ++r) part[r] = 0.f;
+      for (int d = 0; d < D; d += 4) {
+        float k4[4];
+        ldv<A, 4>(kr + d, k4);
+#pragma unroll
+        for (int r = 0; r < kFastMaxRep; ++r) {
+          if (r < rep) {
+            const float4 q4 = *reinterpret_cast<const float4*>(
+                qs + (kv * rep + r) * D + d);
+            part[r] += q4.x * k4[0] + q4.y * k4[1] + q4.z * k4[2] +
+                       q4.w * k4[3];
+          }
+        }
+      }
+      // hand the group's scores to their (statically indexed) slots
+#pragma unroll
+      for (int g = 0; g < MAXH; ++g) {
+        const int r = g - kv * rep;
+        if (g < H && r >= 0 && r < rep) {
+          float pv = part[0];
+#pragma unroll
+          for (int rr = 1; rr < kFastMaxRep; ++rr)
+            if (rr == r) pv = part[rr];
+          raw[g] = pv * scale - r1[g] * log1pf(r2[g] * dist);
+        }
+      }
+    }
+  }
+  // mixing, per-head maxima over the pass
+  float mh[MAXH];
+#pragma unroll
+  for (int h = 0; h < MAXH; ++h) {
+    mh[h] = -INFINITY;
+    if (h < H) {
+      if (live) {
+        float m = 0.f;
+#pragma unroll
+        for (int g = 0; g < MAXH; ++g)
+          if (g < H) m += tk[h * H + g] * raw[g];
+        mh[h] = m;
+      }
+      const float wm = wave_reduce_max(mh[h]);
+      if (lane == 0) wred[wave * H + h] = wm;
+    }
+  }
+  __syncthreads();
+  float wsum[MAXH];
+#pragma unroll
+  for (int h = 0; h < MAXH; ++h) {
+    if (h < H) {
+      // finite: key j0 is live
+      const float mt = fmaxf(fmaxf(wred[h], wred[H + h]),
+                             fmaxf(wred[2 * H + h], wred[3 * H + h]));
+      const float pw = live ? expf(mh[h] - mt) : 0.f;
+      pbuf[h * kFastKT + tid] = pw;
+      wsum[h] = wave_reduce_sum(pw);
+      if (tid == 0) pml[h] = mt;
+    }
+  }
+  __syncthreads();       // everyone has read the maxima; weights are in LDS
+#pragma unroll
+  for (int h = 0; h < MAXH; ++h)
+    if (h < H && lane == 0) wred[wave * H + h] = wsum[h];
+  const int nk = min(kFastKT, p - j0 + 1);
+#pragma unroll
+  for (int x = 0; x < kFastItems; ++x) {
+    const int it = tid + 256 * x;
+    if (it < nitems) {
+      const int h = it / (V / 4), c = (it % (V / 4)) * 4;
+      float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+      const float* pw = pbuf + h * kFastKT;
+      const int kvh = h / rep;
+      for (int jj = 0; jj < nk; ++jj) {
+        const int jk = j0 + jj;
+        const int64_t blk = bt[jk / bs];
+        float v4[4];
+        ldv<A, 4>(v_cache + ((blk * G + kvh) * bs + jk % bs) * V + c, v4);
+        const float w = pw[jj];
+        a0 += w * v4[0];
+        a1 += w * v4[1];
+        a2 += w * v4[2];
+        a3 += w * v4[3];
+      }
+      *reinterpret_cast<float4*>(po + h * V + c) = float4{a0, a1, a2, a3};
+    }
+  }
+  __syncthreads();
+  if (tid < H)
+    pml[H + tid] = wred[tid] + wred[H + tid] + wred[2 * H + tid] +
+                   wred[3 * H + tid];
+}
+
+// out[h][c] = sum_s e^(m_s - M) o_s[h][c] / sum_s e^(m_s - M) l_s
+template <typename A>
+__global__ __launch_bounds__(256) void talking_window_combine_kernel(
+    A* __restrict__ out, const float* __restrict__ part_ml,
+    const float* __restrict__ part_o, int row_begin, int nsplit, int H,
+    int V) {
+  const int64_t r = blockIdx.x;
+  const float* ml = part_ml + r * nsplit * 2 * H;
+  const float* po = part_o + r * nsplit * H * V;
+  for (int o = threadIdx.x; o < H * V; o += 256) {
+    const int h = o / V;
+    float M = -INFINITY;
+    for (int sp = 0; sp < nsplit; ++sp) M = fmaxf(M, ml[sp * 2 * H + h]);
+    float num = 0.f, den = 0.f;
+    for (int sp = 0; sp < nsplit; ++sp) {
+      const float m = ml[sp * 2 * H + h];
+      if (m == -INFINITY) continue;
+      const float f = expf(m - M);
+      num += f * po[static_cast<int64_t>(sp) * H * V + o];
+      den += f * ml[sp * 2 * H + H + h];
+    }
+    Act<A>::st(out + (row_begin + r) * H * V + o, num / den);
+  }
+}
+
 typedef __attribute__((ext_vector_type(4))) short short4v;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
@@ -274,6 +461,12 @@ __global__ __launch_bounds__(256) void talking_window_tile_kernel(
 #pragma unroll
     for (int vb = 0; vb < VB; ++vb) o[qs][vb] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
+  // short groups (a decoded row is a group of one): waves and query sets
+  // without rows only help staging (wave-uniform flags)
+  bool set_on[QS];
+#pragma unroll
+  for (int qs = 0; qs < QS; ++qs) set_on[qs] = (wave * QS + qs) * 16 < nrows;
+  const bool wave_on = set_on[0];
 
   for (int j0 = kv_lo; j0 <= kv_hi; j0 += BN) {
     floatx4 sacc[QS][NB];
@@ -341,7 +534,9 @@ __global__ __launch_bounds__(256) void talking_window_tile_kernel(
       __syncthreads();
 
       // ---- S^T += K_kv Q'_kv^T ----
-      if constexpr (BF) {
+      if (!wave_on) {
+        // nothing to compute for this wave
+      } else if constexpr (BF) {
         short4v qfr[QS][DB];
 #pragma unroll
         for (int qs = 0; qs < QS; ++qs)
@@ -360,8 +555,9 @@ __global__ __launch_bounds__(256) void talking_window_tile_kernel(
                 *reinterpret_cast<const short4v*>(kr + 16 * kk + 4 * g4);
 #pragma unroll
             for (int qs = 0; qs < QS; ++qs)
-              sacc[qs][nb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
-                  a, qfr[qs][kk], sacc[qs][nb], 0, 0, 0);
+              if (set_on[qs])
+                sacc[qs][nb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+                    a, qfr[qs][kk], sacc[qs][nb], 0, 0, 0);
           }
         }
       } else {
@@ -376,8 +572,9 @@ __global__ __launch_bounds__(256) void talking_window_tile_kernel(
             const float a = k_lds[(nb * 16 + c16) * KP + 4 * kk + g4];
 #pragma unroll
             for (int qs = 0; qs < QS; ++qs)
-              sacc[qs][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                  a, qv[qs], sacc[qs][nb], 0, 0, 0);
+              if (set_on[qs])
+                sacc[qs][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                    a, qv[qs], sacc[qs][nb], 0, 0, 0);
           }
         }
       }
@@ -386,6 +583,10 @@ __global__ __launch_bounds__(256) void talking_window_tile_kernel(
     }
 
     // ---- scale, distance penalty, mask, online softmax ----
+    if (!wave_on) {
+      __syncthreads();
+      continue;
+    }
     float sv[QS][NB][4];
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs) {
@@ -443,8 +644,9 @@ __global__ __launch_bounds__(256) void talking_window_tile_kernel(
               *reinterpret_cast<const short4v*>(vr + nb * 16 + 4 * g4);
 #pragma unroll
           for (int qs = 0; qs < QS; ++qs)
-            o[qs][vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
-                a, pf[qs][nb], o[qs][vb], 0, 0, 0);
+            if (set_on[qs])
+              o[qs][vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+                  a, pf[qs][nb], o[qs][vb], 0, 0, 0);
         }
       }
     } else {
@@ -457,8 +659,9 @@ __global__ __launch_bounds__(256) void talking_window_tile_kernel(
             const float a = v_lds[(nb * 16 + 4 * g4 + i) * VP + vb * 16 + c16];
 #pragma unroll
             for (int qs = 0; qs < QS; ++qs)
-              o[qs][vb] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                  a, sv[qs][nb][i], o[qs][vb], 0, 0, 0);
+              if (set_on[qs])
+                o[qs][vb] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                    a, sv[qs][nb][i], o[qs][vb], 0, 0, 0);
           }
     }
     __syncthreads();
@@ -479,6 +682,23 @@ __global__ __launch_bounds__(256) void talking_window_tile_kernel(
 
 }  // namespace
 
+size_t talking_window_fast_smem(int H, int D) {
+  return sizeof(float) *
+         (static_cast<size_t>(H) * D + H * kFastKT + H * H + 4 * H);
+}
+
+// sizes the thread-per-key row kernel handles
+bool talking_window_fast_fits(int H, int G, int D, int V) {
+  return D % 4 == 0 && V % 4 == 0 && H <= 32 && H / G <= kFastMaxRep &&
+         H * V / 4 <= 256 * kFastItems &&
+         talking_window_fast_smem(H, D) <= 64 * 1024;
+}
+
+// key passes (workgroups per row) for a visible range of at most max_keys
+int talking_window_fast_splits(int max_keys) {
+  return max(ceil_div(max_keys, kFastKT), 1);
+}
+
 size_t talking_window_row_smem(int H, int D) {
   return sizeof(float) *
          (static_cast<size_t>(H) * D + 2 * H * kRowKT + H * H + 5 * H);
@@ -492,8 +712,29 @@ void launch_talking_window_rows(A* out, const A* q, int64_t q_stride,
                                 const float* r1, const float* r2,
                                 const float* talk, int row_begin, int rows,
                                 int H, int G, int D, int V, int bs,
-                                float scale, int window, hipStream_t st) {
+                                float scale, int window, float* part_ml,
+                                float* part_o, int nsplit, hipStream_t st) {
   if (rows <= 0) return;
+  // thread-per-key form where 4-wide accesses and the register budget fit
+  if (talking_window_fast_fits(H, G, D, V) && part_ml != nullptr) {
+    const size_t fast_smem = talking_window_fast_smem(H, D);
+    const dim3 grid(rows, nsplit);
+    if (H <= 16)
+      hipLaunchKernelGGL((talking_window_row_fast_kernel<A, 16>), grid,
+                         dim3(256), fast_smem, st, part_ml, part_o, q,
+                         q_stride, k_cache, v_cache, seq_bt, bt_width, row_seq,
+                         positions, r1, r2, talk, row_begin, H, G, D, V, bs,
+                         scale, window);
+    else
+      hipLaunchKernelGGL((talking_window_row_fast_kernel<A, 32>), grid,
+                         dim3(256), fast_smem, st, part_ml, part_o, q,
+                         q_stride, k_cache, v_cache, seq_bt, bt_width, row_seq,
+                         positions, r1, r2, talk, row_begin, H, G, D, V, bs,
+                         scale, window);
+    hipLaunchKernelGGL(talking_window_combine_kernel<A>, dim3(rows), dim3(256),
+                       0, st, out, part_ml, part_o, row_begin, nsplit, H, V);
+    return;
+  }
   const size_t smem = talking_window_row_smem(H, D);
   const int per = ceil_div(H * V, 256);
 #define FI_LAUNCH(N)                                                          \
@@ -573,7 +814,7 @@ bool launch_talking_window_tiles(A* out, A* qf, float* pen, int maxd,
   template void launch_talking_window_rows<A>(                                \
       A*, const A*, int64_t, const A*, const A*, const int*, int, const int*, \
       const int*, const float*, const float*, const float*, int, int, int,    \
-      int, int, int, int, float, int, hipStream_t);
+      int, int, int, int, float, int, float*, float*, int, hipStream_t);
 FI_INST(float)
 FI_INST(u16)
 #undef FI_INST

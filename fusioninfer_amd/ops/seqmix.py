@@ -292,12 +292,25 @@ def talking_window_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
             maxd = int(window) if window > 0 else seq_bt.shape[1] * bs
             pen = torch.empty((heads, maxd), dtype=torch.float32,
                               device=q.device)
+        part_ml = part_o = None
+        rest = T - tile_rows
+        if rest > 0:
+            # rows outside the tile table (decoded rows): one partial
+            # result per 256-key pass of the visible range
+            bs = k_cache.shape[2]
+            keys = int(window) if window > 0 else seq_bt.shape[1] * bs
+            ns = _native().talking_window_splits(keys)
+            V = v_cache.shape[3]
+            part_ml = torch.empty((rest, ns, 2, heads), dtype=torch.float32,
+                                  device=q.device)
+            part_o = torch.empty((rest, ns, heads * V), dtype=torch.float32,
+                                 device=q.device)
         _native().talking_window_attention(out, q, k_cache, v_cache, seq_bt,
                                            row_seq, positions, float(scale),
                                            int(window), r1, r2, talk,
                                            int(heads), seq_cu, tile_seq,
                                            tile_row0, int(tile_rows), folded,
-                                           pen)
+                                           pen, part_ml, part_o)
         return out
     return ref.talking_window_attention(
         q.reshape(T, heads, dim), k_cache, v_cache, seq_bt, row_seq,
