@@ -198,6 +198,7 @@ __global__ __launch_bounds__(256) void talking_window_row_fast_kernel(
   float* pbuf = qs + H * D;              // [H][KT] weights of this pass
   float* tk = pbuf + H * kFastKT;        // [H][H]
   float* wred = tk + H * H;              // [4][H] per-wave partials
+  int* kblk = reinterpret_cast<int*>(wred + 4 * H);   // [KT] key's row base
 
   const int t = row_begin + blockIdx.x;
   const int split = blockIdx.y, nsplit = gridDim.y;
@@ -234,12 +235,15 @@ __global__ __launch_bounds__(256) void talking_window_row_fast_kernel(
   for (int g = 0; g < MAXH; ++g) raw[g] = 0.f;
   if (live) {
     const int64_t blk = bt[j / bs];
+    // row index of kv head 0 of this key; head kv adds kv * bs rows
+    kblk[tid] = static_cast<int>(blk * G * bs + j % bs);
     const float dist = static_cast<float>(p - j);
     for (int kv = 0; kv < G; ++kv) {
       const A* kr = k_cache + ((blk * G + kv) * bs + j % bs) * D;
       float part[kFastMaxRep];
 #pragma unroll
       for (int r = 0; r < kFastMaxRep; ++r) part[r] = 0.f;
+#pragma unroll 4
       for (int d = 0; d < D; d += 4) {
         float k4[4];
         ldv<A, 4>(kr + d, k4);
@@ -310,12 +314,11 @@ __global__ __launch_bounds__(256) void talking_window_row_fast_kernel(
       const int h = it / (V / 4), c = (it % (V / 4)) * 4;
       float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
       const float* pw = pbuf + h * kFastKT;
-      const int kvh = h / rep;
+      const A* vbase = v_cache + static_cast<int64_t>(h / rep) * bs * V + c;
+#pragma unroll 4
       for (int jj = 0; jj < nk; ++jj) {
-        const int jk = j0 + jj;
-        const int64_t blk = bt[jk / bs];
         float v4[4];
-        ldv<A, 4>(v_cache + ((blk * G + kvh) * bs + jk % bs) * V + c, v4);
+        ldv<A, 4>(vbase + static_cast<int64_t>(kblk[jj]) * V, v4);
         const float w = pw[jj];
         a0 += w * v4[0];
         a1 += w * v4[1];
@@ -683,8 +686,8 @@ __global__ __launch_bounds__(256) void talking_window_tile_kernel(
 }  // namespace
 
 size_t talking_window_fast_smem(int H, int D) {
-  return sizeof(float) *
-         (static_cast<size_t>(H) * D + H * kFastKT + H * H + 4 * H);
+  return sizeof(float) * (static_cast<size_t>(H) * D + H * kFastKT + H * H +
+                          4 * H + kFastKT);
 }
 
 // sizes the thread-per-key row kernel handles
