@@ -340,7 +340,7 @@ class DecayLinearAttention(nn.Module):
         c = self.cfg
         o_raw = seqmix.decay_linear_attention(
             q, k, v, self.decay, cache["lin"], meta.seq_cu, meta.seq_slots,
-            meta.positions, c.heads, c.dim, c.vdim)
+            meta.positions, c.heads, c.dim, c.vdim, row_seq=meta.row_seq)
         o = seqmix.group_rms_gate(o_raw, g, self.norm_w, 1, self.eps,
                                   "sigmoid", self.dtype)
         return self.o_proj(o)
@@ -486,17 +486,27 @@ class RoutedExperts(nn.Module):
                 and self.ff % 64 == 0 and self.experts <= 128)
 
     def invalidate_packed(self):
-        self._packed = None
+        """The expert weights changed (checkpoint load, tests): repack on
+        next use."""
+        self._packed_stale = True
 
     def _packed_weights(self):
-        if self._packed is None:
+        if self._packed is None or getattr(self, "_packed_stale", False):
             from fusioninfer_amd import ops
 
-            self._packed = (
+            fresh = (
                 ops.pack_moe_weights(
                     self.gate_up.data.transpose(1, 2).contiguous()),
                 ops.pack_moe_weights(
                     self.down.data.transpose(1, 2).contiguous()))
+            if self._packed is None:
+                self._packed = fresh
+            else:
+                # in place: captured decode graphs keep reading these
+                # tensors
+                for old, new in zip(self._packed, fresh):
+                    old.copy_(new)
+            self._packed_stale = False
         return self._packed
 
     def route(self, x):

@@ -47,6 +47,7 @@ SEQMIX_SOURCES = [
     "seqmix_attention.hip",
     "seqmix_delta.hip",
     "seqmix_stream.hip",
+    "seqmix_linear.hip",
     "seqmix_window.hip",
 ]
 

@@ -68,8 +68,8 @@ template <typename A>
 void launch_decay_linear_attention(float*, float*, float*, const A*, const A*,
                                    const A*, int64_t, int64_t, int64_t,
                                    const float*, float*, const int*,
-                                   const int*, const int*, int, int, int, int,
-                                   int, bool, hipStream_t);
+                                   const int*, const int*, const int*, int,
+                                   int, int, int, int, bool, hipStream_t);
 template <typename A>
 void launch_gated_delta_rule(float*, float*, float*, const A*, int64_t,
                              const float*, const A*, int64_t, const A*,
@@ -530,7 +530,8 @@ void decay_linear_attention(at::Tensor o_raw, at::Tensor vecs, at::Tensor vbuf,
                             at::Tensor decay, at::Tensor state,
                             at::Tensor seq_cu, at::Tensor seq_slots,
                             at::Tensor positions, int64_t heads, int64_t dim,
-                            int64_t vdim, bool silu) {
+                            int64_t vdim, bool silu,
+                            c10::optional<at::Tensor> row_seq) {
   CHECK_ACT(q);
   const int64_t T = q.size(0);
   TORCH_CHECK(k.is_cuda() && v.is_cuda() &&
@@ -547,13 +548,19 @@ void decay_linear_attention(at::Tensor o_raw, at::Tensor vecs, at::Tensor vbuf,
               state.size(2) == dim && state.size(3) == vdim);
   check_groups(seq_cu, seq_slots, positions, T);
   const int S = seq_slots.numel();
+  const int* rs = nullptr;
+  if (row_seq.has_value()) {
+    CHECK_I32(*row_seq);
+    TORCH_CHECK(row_seq->numel() == T);
+    rs = row_seq->data_ptr<int>();
+  }
   DISPATCH_ACT(q, fi::launch_decay_linear_attention<A>(
                       o_raw.data_ptr<float>(), vecs.data_ptr<float>(),
                       vbuf.data_ptr<float>(), ptr<A>(q), ptr<A>(k), ptr<A>(v),
                       q.stride(0), k.stride(0), v.stride(0),
                       decay.data_ptr<float>(), state.data_ptr<float>(),
                       seq_cu.data_ptr<int>(), seq_slots.data_ptr<int>(),
-                      positions.data_ptr<int>(), (int)T, S, (int)heads,
+                      positions.data_ptr<int>(), rs, (int)T, S, (int)heads,
                       (int)dim, (int)vdim, silu, stream()));
 }
 

@@ -104,7 +104,8 @@ __global__ __launch_bounds__(64 * kDeltaWaves) void delta_rule_wave_kernel(
     const float* __restrict__ vecs,             // [T, heads, 5, DK]
     const A* __restrict__ v, int64_t v_stride, float* __restrict__ state,
     const int* __restrict__ seq_cu, const int* __restrict__ seq_slots,
-    const int* __restrict__ positions, int heads, int dim, int vdim) {
+    const int* __restrict__ positions, int heads, int dim, int vdim,
+    int max_rows) {
   constexpr int RS = DK / SL;      // rows per lane
   constexpr int R4 = RS / 4;
   constexpr int COLS = 64 / SL;    // columns per wave
@@ -122,7 +123,8 @@ __global__ __launch_bounds__(64 * kDeltaWaves) void delta_rule_wave_kernel(
   const int head = blockIdx.y;
   const int s = blockIdx.z;
   const int row0 = seq_cu[s], row1 = seq_cu[s + 1];
-  if (row1 <= row0) return;
+  // longer groups may belong to another kernel (chunk-parallel forms)
+  if (row1 <= row0 || row1 - row0 > max_rows) return;
   const int slot = seq_slots[s];
   const bool col_ok = c < vdim;
   const int hbase = head * vdim;
@@ -283,14 +285,15 @@ template <typename VT>
 void launch_recurrence(float* o_raw, const float* vecs, const VT* v,
                        int64_t v_stride, float* state, const int* seq_cu,
                        const int* seq_slots, const int* positions, int S,
-                       int heads, int dim, int vdim, hipStream_t st) {
+                       int heads, int dim, int vdim, hipStream_t st,
+                       int max_rows = 0x7fffffff) {
   const int DK = delta_row_capacity(dim);
 #define FI_LAUNCH(DKK, SL, TB)                                                 \
   hipLaunchKernelGGL(                                                          \
       (delta_rule_wave_kernel<VT, DKK, SL, TB>),                               \
       dim3(ceil_div(vdim, kDeltaWaves * 64 / SL), heads, S),                   \
       dim3(64 * kDeltaWaves), 0, st, o_raw, vecs, v, v_stride, state, seq_cu,  \
-      seq_slots, positions, heads, dim, vdim)
+      seq_slots, positions, heads, dim, vdim, max_rows)
   if (DK == 64) {
     FI_LAUNCH(64, 8, 8);
   } else if (DK == 128) {
@@ -367,6 +370,15 @@ __global__ __launch_bounds__(256) void decay_linear_prep_kernel(
   }
 }
 
+bool launch_decay_linear_chunks(float*, const float*, int, const float*,
+                                const float*, float*, const int*, const int*,
+                                const int*, int, int, int, int, int,
+                                hipStream_t);
+
+// The preparation kernel runs for every row; groups of two or more rows
+// (prompt portions) then take the chunk-parallel kernel where the key size
+// has a variant and the row -> group map is given, one-row groups (decoded
+// tokens) and everything else the serial recurrence.
 template <typename A>
 void launch_decay_linear_attention(float* o_raw, float* vecs, float* vbuf,
                                    const A* q, const A* k, const A* v,
@@ -374,8 +386,9 @@ void launch_decay_linear_attention(float* o_raw, float* vecs, float* vbuf,
                                    int64_t v_stride, const float* decay,
                                    float* state, const int* seq_cu,
                                    const int* seq_slots, const int* positions,
-                                   int T, int S, int heads, int dim, int vdim,
-                                   bool silu, hipStream_t st) {
+                                   const int* row_seq, int T, int S, int heads,
+                                   int dim, int vdim, bool silu,
+                                   hipStream_t st) {
   if (S == 0 || T == 0) return;
   const int64_t items = static_cast<int64_t>(T) * heads;
   const int nblk = static_cast<int>((items + 3) / 4);
@@ -383,9 +396,16 @@ void launch_decay_linear_attention(float* o_raw, float* vecs, float* vbuf,
   hipLaunchKernelGGL(decay_linear_prep_kernel<A>, dim3(nblk), dim3(256), 0, st,
                      vecs, vbuf, q, k, v, q_stride, k_stride, v_stride, decay,
                      T, heads, dim, vdim, DK, silu);
+  int max_rows = 0x7fffffff;
+  if (row_seq != nullptr && T > S &&
+      launch_decay_linear_chunks(o_raw, vecs, DK, vbuf, decay, state, seq_cu,
+                                 seq_slots, positions, S, heads, dim, vdim, 2,
+                                 st))
+    max_rows = 1;
   launch_recurrence<float>(o_raw, vecs, vbuf,
                            static_cast<int64_t>(heads) * vdim, state, seq_cu,
-                           seq_slots, positions, S, heads, dim, vdim, st);
+                           seq_slots, positions, S, heads, dim, vdim, st,
+                           max_rows);
 }
 
 // ---------------------------------------------------------------------
@@ -574,8 +594,8 @@ FI_INST(u16)
 #define FI_INST(A)                                                             \
   template void launch_decay_linear_attention<A>(                              \
       float*, float*, float*, const A*, const A*, const A*, int64_t, int64_t,  \
-      int64_t, const float*, float*, const int*, const int*, const int*, int,  \
-      int, int, int, int, bool, hipStream_t);                                  \
+      int64_t, const float*, float*, const int*, const int*, const int*,       \
+      const int*, int, int, int, int, int, bool, hipStream_t);                 \
   template void launch_gated_delta_rule<A>(                                    \
       float*, float*, float*, const A*, int64_t, const float*, const A*,       \
       int64_t, const A*, int64_t, const float*, const float*, float*, float*,  \

@@ -229,10 +229,11 @@ def _recurrence_scratch(T: int, heads: int, dim: int, device):
 
 def decay_linear_attention(q, k, v, decay, state, seq_cu, seq_slots,
                            positions, heads: int, dim: int, vdim: int,
-                           silu: bool = True):
+                           silu: bool = True, row_seq=None):
     """Raw fp32 read-outs [T, heads*vdim] of linear attention with one
     scalar decay per head; q/k/v may be column slices of one projection
-    output."""
+    output. With ``row_seq`` (group of every row) the GPU path runs
+    multi-row groups through the chunk-parallel kernel."""
     if q.is_cuda:
         T = q.shape[0]
         o_raw = torch.empty((T, heads * vdim), dtype=torch.float32,
@@ -242,7 +243,8 @@ def decay_linear_attention(q, k, v, decay, state, seq_cu, seq_slots,
                            device=q.device)
         _native().decay_linear_attention(o_raw, vecs, vbuf, q, k, v, decay,
                                          state, seq_cu, seq_slots, positions,
-                                         heads, dim, vdim, bool(silu))
+                                         heads, dim, vdim, bool(silu),
+                                         row_seq)
         return o_raw
     return ref.decay_linear_attention(q, k, v, decay, state, seq_cu,
                                       seq_slots, positions, heads, dim, vdim,

@@ -208,7 +208,8 @@ def _lightning_case(device, heads, dim, vdim, decay, spans, T, boost=None,
         o_raw = seqmix.decay_linear_attention(
             f(hh @ P["q"].T), f(hh @ P["k"].T), f(hh @ P["v"].T), dec, state,
             mk([0, b - a], device), mk([2], device),
-            mk(list(range(a, b)), device), heads, dim, vdim)
+            mk(list(range(a, b)), device), heads, dim, vdim,
+            row_seq=mk([0] * (b - a), device))
         outs.append(seqmix.group_rms_gate(
             o_raw, f(hh @ P["g"].T), f(P["norm"]), 1, 1e-3, "sigmoid",
             torch.float32))
@@ -219,12 +220,20 @@ def _lightning_case(device, heads, dim, vdim, decay, spans, T, boost=None,
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("heads,dim,vdim,decay", [
     (3, 8, 12, (0.5, 0.9, 0.995)), (1, 40, 8, (1.0,)),
-    (2, 72, 136, (0.97, 0.2))])
+    (2, 72, 136, (0.97, 0.2)), (2, 16, 24, (0.9, 0.0)),
+    (2, 32, 80, (1.0, 0.6)), (3, 64, 64, (0.999, 0.97, 0.3)),
+    (2, 128, 144, (0.98, 0.75))])
 def test_decayed_linear_attention_carries_state(device, heads, dim, vdim,
                                                 decay):
     spans = [(0, 1), (1, 9), (9, 10), (10, 12), (12, 30)]
     got, want = _lightning_case(device, heads, dim, vdim, decay, spans, 30)
     assert (got - want).abs().max() < 5e-5
+    # portions longer than one chunk of the chunk-parallel kernel, cut
+    # inside chunks
+    spans = [(0, 70), (70, 73), (73, 74), (74, 201), (201, 230)]
+    got, want = _lightning_case(device, heads, dim, vdim, decay, spans, 230,
+                                seed=1)
+    assert (got - want).abs().max() < 1e-4 * max(1.0, want.abs().max())
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -480,6 +489,24 @@ def test_routed_experts_bf16_gpu(width, ff, E, top, T):
     got, want = _experts_case("cuda", torch.bfloat16, width, ff, E, top, T,
                               seed=2)
     assert rel_err(got, want) < 0.03
+
+
+@pytest.mark.gpu
+def test_repacked_expert_weights_keep_their_storage():
+    """Captured decode graphs read the packed expert tensors: a reload of
+    the weights must refill them in place."""
+    torch.manual_seed(0)
+    with torch.device("cuda"):
+        mod = RoutedExperts(128, 64, 4, 2, torch.bfloat16, scale=1.0)
+    x = torch.randn(9, 128, device="cuda").to(torch.bfloat16)
+    y0 = mod(x)
+    ptrs = [t.data_ptr() for t in mod._packed]
+    mod.gate_up.data.mul_(-0.5)
+    mod.invalidate_packed()
+    y1 = mod(x)
+    assert [t.data_ptr() for t in mod._packed] == ptrs
+    # silu(-g/2) * (-u/2) differs from silu(g) * u: the new weights are used
+    assert (y1.float() - y0.float()).abs().max() > 1e-4
 
 
 # ----------------------------------------------------- model through engine
