@@ -486,23 +486,34 @@ __global__ __launch_bounds__(256) void gated_delta_prep_kernel(
   const float sp = z > 20.f ? z : log1pf(expf(z));
   const float g = expf(-expf(a_log[head]) * sp);
 
+  // convolved q/k of this lane's rows (DK <= 256: at most four per lane),
+  // evaluated once
+  float qc[4], kc[4];
   float qsq = 0.f, ksq = 0.f;
-  for (int i = lane; i < dim; i += 64) {
-    const float qv = cs.at(kvh * dim + i);
-    const float kv = cs.at(nq + kvh * dim + i);
-    qsq += qv * qv;
-    ksq += kv * kv;
+#pragma unroll
+  for (int x = 0; x < 4; ++x) {
+    const int i = lane + 64 * x;
+    qc[x] = kc[x] = 0.f;
+    if (i < dim) {
+      qc[x] = cs.at(kvh * dim + i);
+      kc[x] = cs.at(nq + kvh * dim + i);
+      qsq += qc[x] * qc[x];
+      ksq += kc[x] * kc[x];
+    }
   }
   qsq = wave_reduce_sum(qsq);
   ksq = wave_reduce_sum(ksq);
   const float qinv = rsqrtf(qsq + 1e-6f) * rsqrtf(static_cast<float>(dim));
   const float kinv = rsqrtf(ksq + 1e-6f);
   float* dst = vecs + item * 5 * DK;
-  for (int i = lane; i < DK; i += 64) {
+#pragma unroll
+  for (int x = 0; x < 4; ++x) {
+    const int i = lane + 64 * x;
+    if (i >= DK) break;
     float ww = 1.f, au = 0.f, uu = 0.f, rr = 0.f;
     if (i < dim) {
-      uu = cs.at(nq + kvh * dim + i) * kinv;
-      rr = cs.at(kvh * dim + i) * qinv;
+      uu = kc[x] * kinv;
+      rr = qc[x] * qinv;
       ww = g;
       au = beta * g * uu;
     }
