@@ -171,19 +171,20 @@ __global__ __launch_bounds__(256) void talking_window_row_kernel(
 
 
 // Row kernel, thread-per-key form (decode rows when the sizes allow 4-wide
-// accesses): 256 keys per pass, one per thread. A thread reads its key's
+// accesses): 64 keys per wave and pass, one per thread. A thread reads its key's
 // rows of all kv heads once (vector loads), forms the raw scores of all
 // heads against the query held in LDS (broadcast reads), mixes them in
 // registers, and the block then takes per-head maxima and sums across
 // threads (wave shuffles + one LDS hop). For the weighted value sum the
 // threads switch to owning (head, 4 value columns) outputs and walk the
 // pass's weights in LDS.
-constexpr int kFastKT = 256;
+constexpr int kFastWaves = 4;       // waves per workgroup of the fast row kernel
+constexpr int kFastKT = 64 * kFastWaves;
 constexpr int kFastMaxRep = 8;
 constexpr int kFastItems = 4;      // (head, 4 columns) outputs per thread
 
 template <typename A, int MAXH>
-__global__ __launch_bounds__(256) void talking_window_row_fast_kernel(
+__global__ __launch_bounds__(kFastKT) void talking_window_row_fast_kernel(
     float* __restrict__ part_ml,         // [rows, nsplit, 2, H] max, sum
     float* __restrict__ part_o,          // [rows, nsplit, H*V]
     const A* __restrict__ q, int64_t q_stride,
@@ -197,8 +198,8 @@ __global__ __launch_bounds__(256) void talking_window_row_fast_kernel(
   float* qs = smem;                      // [H*D]
   float* pbuf = qs + H * D;              // [H][KT] weights of this pass
   float* tk = pbuf + H * kFastKT;        // [H][H]
-  float* wred = tk + H * H;              // [4][H] per-wave partials
-  int* kblk = reinterpret_cast<int*>(wred + 4 * H);   // [KT] key's row base
+  float* wred = tk + H * H;              // [waves][H] per-wave partials
+  int* kblk = reinterpret_cast<int*>(wred + kFastWaves * H);   // [KT] key's row base
 
   const int t = row_begin + blockIdx.x;
   const int split = blockIdx.y, nsplit = gridDim.y;
@@ -214,7 +215,7 @@ __global__ __launch_bounds__(256) void talking_window_row_fast_kernel(
   float* pml = part_ml + pslot * 2 * H;
   float* po = part_o + pslot * H * V;
 
-  // this workgroup's 256 keys
+  // the keys of this pass, one per thread
   const int j0 = lo + split * kFastKT;
   if (j0 > p) {                          // nothing to see: an empty partial
     if (tid < H) {
@@ -223,9 +224,9 @@ __global__ __launch_bounds__(256) void talking_window_row_fast_kernel(
     }
     return;
   }
-  for (int i = tid; i < H * D; i += 256)
+  for (int i = tid; i < H * D; i += kFastKT)
     qs[i] = Act<A>::ld(q + t * q_stride + i);
-  for (int i = tid; i < H * H; i += 256) tk[i] = talk[i];
+  for (int i = tid; i < H * H; i += kFastKT) tk[i] = talk[i];
   __syncthreads();
 
   const int j = j0 + tid;
@@ -294,8 +295,9 @@ __global__ __launch_bounds__(256) void talking_window_row_fast_kernel(
   for (int h = 0; h < MAXH; ++h) {
     if (h < H) {
       // finite: key j0 is live
-      const float mt = fmaxf(fmaxf(wred[h], wred[H + h]),
-                             fmaxf(wred[2 * H + h], wred[3 * H + h]));
+      float mt = wred[h];
+#pragma unroll
+      for (int w = 1; w < kFastWaves; ++w) mt = fmaxf(mt, wred[w * H + h]);
       const float pw = live ? expf(mh[h] - mt) : 0.f;
       pbuf[h * kFastKT + tid] = pw;
       wsum[h] = wave_reduce_sum(pw);
@@ -309,7 +311,7 @@ __global__ __launch_bounds__(256) void talking_window_row_fast_kernel(
   const int nk = min(kFastKT, p - j0 + 1);
 #pragma unroll
   for (int x = 0; x < kFastItems; ++x) {
-    const int it = tid + 256 * x;
+    const int it = tid + kFastKT * x;
     if (it < nitems) {
       const int h = it / (V / 4), c = (it % (V / 4)) * 4;
       float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
@@ -329,9 +331,12 @@ __global__ __launch_bounds__(256) void talking_window_row_fast_kernel(
     }
   }
   __syncthreads();
-  if (tid < H)
-    pml[H + tid] = wred[tid] + wred[H + tid] + wred[2 * H + tid] +
-                   wred[3 * H + tid];
+  if (tid < H) {
+    float l = wred[tid];
+#pragma unroll
+    for (int w = 1; w < kFastWaves; ++w) l += wred[w * H + tid];
+    pml[H + tid] = l;
+  }
 }
 
 // out[h][c] = sum_s e^(m_s - M) o_s[h][c] / sum_s e^(m_s - M) l_s
@@ -687,13 +692,13 @@ __global__ __launch_bounds__(256) void talking_window_tile_kernel(
 
 size_t talking_window_fast_smem(int H, int D) {
   return sizeof(float) * (static_cast<size_t>(H) * D + H * kFastKT + H * H +
-                          4 * H + kFastKT);
+                          kFastWaves * H + kFastKT);
 }
 
 // sizes the thread-per-key row kernel handles
 bool talking_window_fast_fits(int H, int G, int D, int V) {
   return D % 4 == 0 && V % 4 == 0 && H <= 32 && H / G <= kFastMaxRep &&
-         H * V / 4 <= 256 * kFastItems &&
+         H * V / 4 <= kFastKT * kFastItems &&
          talking_window_fast_smem(H, D) <= 64 * 1024;
 }
 
@@ -724,13 +729,13 @@ void launch_talking_window_rows(A* out, const A* q, int64_t q_stride,
     const dim3 grid(rows, nsplit);
     if (H <= 16)
       hipLaunchKernelGGL((talking_window_row_fast_kernel<A, 16>), grid,
-                         dim3(256), fast_smem, st, part_ml, part_o, q,
+                         dim3(kFastKT), fast_smem, st, part_ml, part_o, q,
                          q_stride, k_cache, v_cache, seq_bt, bt_width, row_seq,
                          positions, r1, r2, talk, row_begin, H, G, D, V, bs,
                          scale, window);
     else
       hipLaunchKernelGGL((talking_window_row_fast_kernel<A, 32>), grid,
-                         dim3(256), fast_smem, st, part_ml, part_o, q,
+                         dim3(kFastKT), fast_smem, st, part_ml, part_o, q,
                          q_stride, k_cache, v_cache, seq_bt, bt_width, row_seq,
                          positions, r1, r2, talk, row_begin, H, G, D, V, bs,
                          scale, window);
